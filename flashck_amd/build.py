@@ -1,0 +1,65 @@
+"""In-tree build of the gfx950 FMHA library (libflashck_fmha.so) with hipcc.
+
+``python -m flashck_amd.build`` compiles every translation unit under ``csrc/`` for gfx950 and links the shared
+library next to this file.  hipcc cross-compiles, so no GPU is needed to build.
+"""
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "csrc", "build")
+LIB = os.path.join(HERE, "libflashck_fmha.so")
+
+SOURCES = ["fmha_api.cpp", "splitkv_decode.hip", "splitkv_combine.hip", "appendkv_rope.hip", "prefill.hip"]
+
+FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "--offload-arch=gfx950", "-fno-gpu-rdc",
+    # packed fp32 VALU forms are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the FMHA library cannot be built")
+    return exe
+
+
+def _compile(src, extra):
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    cmd = [hipcc(), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS + extra
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{out}")
+    return obj, out
+
+
+def build(verbose=False, extra_flags=()):
+    os.makedirs(OBJ, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 4)) as ex:
+        results = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
+    objs = [o for o, _ in results]
+    if verbose:
+        for _, out in results:
+            if out.strip():
+                print(out)
+    tmp = LIB + ".tmp"
+    cmd = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-fno-gpu-rdc", "-o", tmp] + objs
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stdout}")
+    os.replace(tmp, LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True, extra_flags=sys.argv[1:]))

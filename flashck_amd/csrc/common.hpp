@@ -1,0 +1,201 @@
+// Shared device/host helpers for the gfx950 FMHA kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fck {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+#define FCK_LDS __attribute__((address_space(3)))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Element traits: storage is 16 bit; MFMA operands are 8 packed elements.
+struct BF16 {
+    typedef bf16x8_t vec8;
+    typedef __bf16 elem;
+    // round to nearest even (v_cvt_pk_bf16_f32 on gfx950)
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        bf2 v;
+        v[0] = (__bf16)lo;
+        v[1] = (__bf16)hi;
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float to_f32(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
+    static __device__ __forceinline__ uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+    static __device__ __forceinline__ f32x4_t mfma16(vec8 a, vec8 b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x16_t mfma32(vec8 a, vec8 b, f32x16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+struct FP16 {
+    typedef f16x8_t vec8;
+    typedef _Float16 elem;
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 v;
+        v[0] = (_Float16)lo;
+        v[1] = (_Float16)hi;
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float to_f32(uint16_t x) { return (float)__builtin_bit_cast(_Float16, x); }
+    static __device__ __forceinline__ uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+    static __device__ __forceinline__ f32x4_t mfma16(vec8 a, vec8 b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x16_t mfma32(vec8 a, vec8 b, f32x16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <typename V>
+__device__ __forceinline__ V as_vec8(u32x4_t x)
+{
+    return __builtin_bit_cast(V, x);
+}
+
+// 16-byte global load through the vector memory path.
+__device__ __forceinline__ u32x4_t ldg16(const void* p) { return *reinterpret_cast<const u32x4_t*>(p); }
+
+// Transposing LDS read: within each group of 16 lanes, lane i receives element (i % 4) of the 8 bytes that lane
+// 4k + i/4 addressed, for k = 0..3.  When lanes 4k..4k+3 address 16 consecutive 16-bit columns of row k, lane i ends up
+// with column i of rows 0..3.
+__device__ __forceinline__ u32x2_t lds_read_tr16(const void FCK_LDS* p)
+{
+    s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t FCK_LDS*)p);
+    return __builtin_bit_cast(u32x2_t, v);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Visible key range [lo, hi) of query row i: GenericAttentionMask::IsOutOfBound,
+// ck_tile/ops/fmha/block/block_masking.hpp:359-373 with (y, x) from
+// make_generic_attention_mask_coordinates_from_lr_window, same file :608-628.
+struct MaskYX {
+    int32_t y, x;  // only read when masking != 0
+    int32_t masking;
+};
+
+__host__ __device__ inline MaskYX make_mask(uint32_t mask_type, int64_t wl, int64_t wr, int32_t sq, int32_t sk)
+{
+    MaskYX m;
+    m.masking = mask_type != 0;
+    const bool tl = mask_type == 1;
+    const int64_t left_tmp = tl ? sq - 1 : sk - 1;
+    const int64_t right_tmp = tl ? sk - 1 : sq - 1;
+    const int64_t l = wl < 0 ? left_tmp : wl;
+    const int64_t r = wr < 0 ? right_tmp : wr;
+    int64_t x = 1 + r + (tl ? 0 : sk - sq);
+    int64_t y = 1 + l + (tl ? 0 : sq - sk);
+    // clamp: only comparisons against [0, sk] matter
+    const int64_t big = (int64_t)1 << 30;
+    x = x > big ? big : (x < -big ? -big : x);
+    y = y > big ? big : (y < -big ? -big : y);
+    m.x = (int32_t)x;
+    m.y = (int32_t)y;
+    return m;
+}
+
+__host__ __device__ inline int32_t mask_lo(const MaskYX& m, int32_t i)
+{
+    if (!m.masking) return 0;
+    const int32_t v = i + 1 - m.y;
+    return v > 0 ? v : 0;
+}
+__host__ __device__ inline int32_t mask_hi(const MaskYX& m, int32_t i, int32_t sk)
+{
+    if (!m.masking) return sk;
+    const int64_t v = (int64_t)i + m.x;
+    return v < sk ? (v > 0 ? (int32_t)v : 0) : sk;
+}
+
+// Where the K/V rows of one sequence live.  `table` == nullptr: rows are contiguous from base_row.
+// Otherwise logical key j sits at row table[j / page] * page + j % page.
+struct KvSeq {
+    const int32_t* table;
+    int64_t base_row;
+    int32_t len;  // number of keys
+};
+
+struct KvAddr {
+    // mode 0: batch cache (+ cache_batch_idx); 1: group; 2: block table; 3: page list
+    int32_t mode;
+    int32_t page_size;
+    int32_t page_shift;  // log2(page_size) when it is a power of two, else -1
+    int32_t seqlen_k;    // batch mode: rows per cache sequence / default key count
+    const int32_t* seqstart_k;
+    const int32_t* seqlen_k_ptr;
+    const int32_t* block_table;
+    int32_t block_table_stride;
+    const int32_t* cache_batch_idx;
+    const int32_t* kv_indptr;
+    const int32_t* kv_page_indices;
+    const int32_t* kv_last_page_lens;
+};
+
+__device__ __forceinline__ KvSeq kv_seq(const KvAddr& a, int b)
+{
+    KvSeq s;
+    if (a.mode == 0) {
+        const int cb = a.cache_batch_idx ? a.cache_batch_idx[b] : b;
+        s.table = nullptr;
+        s.base_row = (int64_t)cb * a.seqlen_k;
+        s.len = a.seqlen_k_ptr ? a.seqlen_k_ptr[b] : a.seqlen_k;
+    } else if (a.mode == 1) {
+        const int s0 = a.seqstart_k[b];
+        s.table = nullptr;
+        s.base_row = s0;
+        s.len = a.seqstart_k[b + 1] - s0;
+    } else if (a.mode == 2) {
+        s.table = a.block_table + (int64_t)b * a.block_table_stride;
+        s.base_row = 0;
+        s.len = a.seqlen_k_ptr[b];
+    } else {
+        const int p0 = a.kv_indptr[b], p1 = a.kv_indptr[b + 1];
+        s.table = a.kv_page_indices + p0;
+        s.base_row = 0;
+        const int np = p1 - p0;
+        const int last = a.kv_last_page_lens ? a.kv_last_page_lens[b] : a.page_size;
+        s.len = np > 0 ? (np - 1) * a.page_size + last : 0;
+    }
+    return s;
+}
+
+__device__ __forceinline__ int64_t kv_row(const KvAddr& a, const KvSeq& s, int j)
+{
+    if (!s.table) return s.base_row + j;
+    int pi, off;
+    if (a.page_shift >= 0) {
+        pi = j >> a.page_shift;
+        off = j & (a.page_size - 1);
+    } else {
+        pi = j / a.page_size;
+        off = j - pi * a.page_size;
+    }
+    return (int64_t)s.table[pi] * a.page_size + off;
+}
+
+}  // namespace fck

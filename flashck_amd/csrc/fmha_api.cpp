@@ -1,0 +1,380 @@
+// Host side of the C ABI declared in include/flashck/fmha/fmha_c_api.h: argument validation, stride / workspace
+// conventions of FlashCK's generated wrappers, kernel selection and launch.  No allocation, no synchronisation.
+#include "flashck/fmha/fmha_c_api.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+
+#include "kernels.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, int32_t dtype, const void* bias)
+{
+    if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16)
+        return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
+    if (batch <= 0 || hq <= 0 || hk <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch and head counts must be positive");
+    if (hq % hk != 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_num_heads %ld is not a multiple of kv_num_heads %ld", (long)hq, (long)hk);
+    if (d != dv) return fail(FCK_ERR_UNSUPPORTED, "qk_head_dim %ld != v_head_dim %ld is not supported", (long)d, (long)dv);
+    if (d != 64 && d != 128 && d != 256) return fail(FCK_ERR_UNSUPPORTED, "head_dim %ld: kernels exist for 64, 128, 256", (long)d);
+    if (bias) return fail(FCK_ERR_UNSUPPORTED, "attention bias / alibi is not supported");
+    return FCK_OK;
+}
+
+int check_mask(uint32_t mask_type)
+{
+    if (mask_type > 3) return fail(FCK_ERR_INVALID_ARGUMENT, "mask_type %u out of range [0,3]", mask_type);
+    return FCK_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int log2_exact(int64_t v)
+{
+    if (v <= 0 || (v & (v - 1))) return -1;
+    int s = 0;
+    while ((int64_t(1) << s) < v) ++s;
+    return s;
+}
+
+int launch_status(hipError_t e, const char* what)
+{
+    if (e != hipSuccess) return fail(FCK_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return FCK_OK;
+}
+
+int cu_count()
+{
+    static int cus = 0;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        int dev = 0;
+        hipDeviceProp_t p;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    });
+    return cus;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* fck_last_error(void) { return g_err; }
+
+const char* fck_fmha_version(void) { return "flashck-fmha-gfx950 0.1"; }
+
+size_t fck_fmha_splitkv_workspace_bytes(int64_t shape_batch, int64_t hq, int64_t shape_sq, int64_t dv, int64_t num_splits)
+{
+    if (shape_batch <= 0 || hq <= 0 || shape_sq <= 0 || dv <= 0 || num_splits <= 0) return 0;
+    const size_t rows = (size_t)shape_batch * hq * num_splits * shape_sq;
+    return rows * dv * sizeof(float) + rows * sizeof(float);
+}
+
+int fck_fmha_num_splits_heuristic(int64_t batch, int64_t hq, int64_t hk, int64_t sq, int64_t max_sk, int64_t head_dim,
+                                  int64_t num_cu)
+{
+    (void)head_dim;
+    if (batch <= 0 || hq <= 0 || hk <= 0 || sq <= 0 || max_sk <= 0) return 1;
+    if (num_cu <= 0) num_cu = cu_count();
+    // One workgroup streams one split of one KV head for 16..64 packed rows (query index x head-in-group).
+    const int64_t g = hq / hk;
+    const int64_t rows = sq * g;
+    const int64_t m_tiles = rows <= 32 ? 1 : (rows + 63) / 64;
+    const int64_t base = batch * hk * m_tiles;  // workgroups without splitting
+    // Aim at >= 2 workgroups per CU so uneven sequence lengths even out, but keep at least 256 keys per split:
+    // below that the merge and the workspace round trip outweigh the streaming.
+    const int64_t want = (2 * num_cu + base - 1) / base;
+    const int64_t cap = max_sk / 256 > 0 ? max_sk / 256 : 1;
+    int64_t ns = want < cap ? want : cap;
+    if (ns < 1) ns = 1;
+    if (ns > 128) ns = 128;
+    return (int)ns;
+}
+
+int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v, const void* bias, void* lse_acc, void* o_acc,
+                         const int32_t* seqstart_q, const int32_t* seqstart_k, const int32_t* seqlen_k_ptr,
+                         const int32_t* block_table, const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
+                         int64_t seqlen_k, int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len,
+                         int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size, float scale,
+                         int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream)
+{
+    g_err[0] = 0;
+    if (int rc = check_common(batch, hq, hk, d, dv, dtype, bias)) return rc;
+    if (int rc = check_mask(mask_type)) return rc;
+    if (!q || !k || !v || !lse_acc || !o_acc) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v, lse_acc and o_acc must not be null");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o_acc))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v and o_acc must be 16-byte aligned");
+    if (num_splits < 1 || num_splits > 128) return fail(FCK_ERR_INVALID_ARGUMENT, "num_splits %ld out of range [1,128]", (long)num_splits);
+    if (!(scale > 0.f) || !std::isfinite(scale)) return fail(FCK_ERR_INVALID_ARGUMENT, "scale must be positive and finite");
+    const bool group = seqstart_q != nullptr;
+    if (!group && seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "seqlen_q must be positive in batch mode");
+    if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
+    if (q_max_seq_len <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_max_seq_len must be positive");
+
+    fck::SplitKvArgs a{};
+    a.q = q;
+    a.k = k;
+    a.v = v;
+    a.o_acc = static_cast<float*>(o_acc);
+    a.lse_acc = static_cast<float*>(lse_acc);
+    a.seqstart_q = seqstart_q;
+    a.batch = (int32_t)batch;
+    a.sq = (int32_t)seqlen_q;
+    a.hq = (int32_t)hq;
+    a.hk = (int32_t)hk;
+    a.num_splits = (int32_t)num_splits;
+    a.shape_sq = seqlen_q;  // group mode: seqlen_q carries total_q (the "shape" length of the FlashCK wrapper)
+    a.scale_log2 = scale * fck::kLog2e;
+    a.mask_type = mask_type;
+    a.window_left = window_left;
+    a.window_right = window_right;
+    if (group && seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "group mode: seqlen_q must carry total_q (workspace row count)");
+
+    bool uniform = true;
+    fck::KvAddr& kv = a.kv;
+    kv.seqlen_k_ptr = seqlen_k_ptr;
+    kv.cache_batch_idx = cache_batch_idx;
+    kv.page_shift = -1;
+    if (block_table) {
+        if (page_block_size <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "paged cache needs page_block_size > 0");
+        if (!seqlen_k_ptr) return fail(FCK_ERR_INVALID_ARGUMENT, "paged cache needs per-sequence key counts (k_seq_len_ptr)");
+        if (max_num_page_blocks < batch || max_num_page_blocks % batch)
+            return fail(FCK_ERR_INVALID_ARGUMENT, "max_num_page_blocks %ld must be a positive multiple of batch %ld", (long)max_num_page_blocks, (long)batch);
+        kv.mode = 2;
+        kv.block_table = block_table;
+        kv.block_table_stride = (int32_t)(max_num_page_blocks / batch);  // fmha_fwd_split_kv_jinja.h:318
+        kv.page_size = (int32_t)page_block_size;
+        kv.page_shift = log2_exact(page_block_size);
+        uniform = page_block_size % 32 == 0;
+    } else if (seqstart_k) {
+        kv.mode = 1;
+        kv.seqstart_k = seqstart_k;
+    } else {
+        if (seqlen_k <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch cache needs seqlen_k > 0");
+        kv.mode = 0;
+        kv.seqlen_k = (int32_t)seqlen_k;
+    }
+    const int rows_max = (int)(q_max_seq_len * (hq / hk));
+    return launch_status(fck::launch_splitkv_decode(a, (int)d, dtype, rows_max, uniform, static_cast<hipStream_t>(stream)),
+                         "FmhaFwdSplitKV launch");
+}
+
+int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o, const int32_t* seqstart_q, int64_t batch,
+                                 int64_t seqlen_q, int64_t hq, int64_t dv, int64_t q_max_seq_len, int64_t num_splits,
+                                 int32_t dtype, void* stream)
+{
+    g_err[0] = 0;
+    (void)q_max_seq_len;
+    if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16)
+        return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
+    if (!lse_acc || !o_acc || !o) return fail(FCK_ERR_INVALID_ARGUMENT, "lse_acc, o_acc and o must not be null");
+    if (batch <= 0 || hq <= 0 || seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch, q_num_heads and seqlen_q must be positive");
+    if (dv != 64 && dv != 128 && dv != 256) return fail(FCK_ERR_UNSUPPORTED, "v_head_dim %ld: kernels exist for 64, 128, 256", (long)dv);
+    if (num_splits < 1 || num_splits > 128) return fail(FCK_ERR_INVALID_ARGUMENT, "num_splits %ld out of range [1,128]", (long)num_splits);
+    if (!aligned16(o_acc) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_acc and o must be 16-byte aligned");
+    fck::CombineArgs a{};
+    a.lse_acc = static_cast<const float*>(lse_acc);
+    a.o_acc = static_cast<const float*>(o_acc);
+    a.o = o;
+    // group mode: one "batch" of total_q rows (seqlen_q carries total_q), fmha_fwd_split_kv_combine_jinja.h:118-119
+    a.Sq = seqlen_q;
+    a.rows = (seqstart_q ? 1 : batch) * seqlen_q;
+    a.hq = (int32_t)hq;
+    a.dv = (int32_t)dv;
+    a.num_splits = (int32_t)num_splits;
+    return launch_status(fck::launch_splitkv_combine(a, dtype, static_cast<hipStream_t>(stream)), "FmhaFwdSplitKVCombine launch");
+}
+
+int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* knew, const void* vnew, const int32_t* seqlen_k,
+                          const int32_t* cu_seqlens_knew, int64_t seqlen_knew, const void* rotary_cos, const void* rotary_sin,
+                          int64_t rotary_dim, int32_t rope_mode, int32_t has_mask, const int32_t* block_table,
+                          int64_t batch_stride_block_table, int64_t page_block_size, const int32_t* cache_batch_idx,
+                          int64_t seqlen_k_cache, int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, int32_t dtype,
+                          void* stream)
+{
+    g_err[0] = 0;
+    if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16)
+        return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
+    if (!k_cache || !v_cache || !knew || !vnew || !seqlen_k) return fail(FCK_ERR_INVALID_ARGUMENT, "k_cache, v_cache, knew, vnew and seqlen_k must not be null");
+    if (batch <= 0 || hk <= 0 || d <= 0 || dv <= 0 || (q && hq <= 0)) return fail(FCK_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    if (d % 2 || dv % 2) return fail(FCK_ERR_INVALID_ARGUMENT, "head dims must be even");
+    if (seqlen_knew <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "seqlen_knew (largest number of new tokens of a sequence) must be positive");
+    if (rope_mode < 0 || rope_mode > 2) return fail(FCK_ERR_INVALID_ARGUMENT, "rope_mode %d out of range [0,2]", rope_mode);
+    if (rope_mode != FCK_ROPE_NONE) {
+        if (!rotary_cos || !rotary_sin) return fail(FCK_ERR_INVALID_ARGUMENT, "rotary tables must not be null when rope_mode != NONE");
+        if (rotary_dim <= 0 || rotary_dim > d || rotary_dim % 2) return fail(FCK_ERR_INVALID_ARGUMENT, "rotary_dim %ld must be even and in (0, %ld]", (long)rotary_dim, (long)d);
+    } else {
+        rotary_dim = 0;
+    }
+    if (block_table) {
+        if (page_block_size <= 0 || batch_stride_block_table <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "paged cache needs page_block_size and batch_stride_block_table > 0");
+    } else if (seqlen_k_cache <= 0) {
+        return fail(FCK_ERR_INVALID_ARGUMENT, "batch cache needs seqlen_k_cache > 0");
+    }
+    fck::AppendKvArgs a{};
+    a.q = q;
+    a.k_cache = k_cache;
+    a.v_cache = v_cache;
+    a.knew = knew;
+    a.vnew = vnew;
+    a.seqlen_k = seqlen_k;
+    a.cu_seqlens_knew = cu_seqlens_knew;
+    a.seqlen_knew = (int32_t)seqlen_knew;
+    a.cos = rotary_cos;
+    a.sin = rotary_sin;
+    a.rotary_dim = (int32_t)rotary_dim;
+    a.rope_mode = rope_mode;
+    a.has_mask = has_mask;
+    a.block_table = block_table;
+    a.block_table_stride = (int32_t)batch_stride_block_table;
+    a.page_size = (int32_t)page_block_size;
+    a.cache_batch_idx = cache_batch_idx;
+    a.seqlen_k_cache = seqlen_k_cache;
+    a.batch = (int32_t)batch;
+    a.hq = (int32_t)hq;
+    a.hk = (int32_t)hk;
+    a.d = (int32_t)d;
+    a.dv = (int32_t)dv;
+    return launch_status(fck::launch_appendkv(a, dtype, (int)seqlen_knew, static_cast<hipStream_t>(stream)), "FmhaFwdAppendKV launch");
+}
+
+static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t q_max_seq_len, bool uniform, void* stream,
+                          const char* what)
+{
+    if (q_max_seq_len <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_max_seq_len must be positive");
+    a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
+    return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+}
+
+int fck_fmha_fwd(const void* q, const void* k, const void* v, const void* bias, void* o, const int32_t* seqstart_q,
+                 const int32_t* seqstart_k, const int32_t* seqlen_k_ptr, int64_t batch, int64_t seqlen_q, int64_t seqlen_k,
+                 int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left,
+                 int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream)
+{
+    g_err[0] = 0;
+    if (int rc = check_common(batch, hq, hk, d, dv, dtype, bias)) return rc;
+    if (int rc = check_mask(mask_type)) return rc;
+    if (!q || !k || !v || !o) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v and o must not be null");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v and o must be 16-byte aligned");
+    if (!(scale > 0.f) || !std::isfinite(scale)) return fail(FCK_ERR_INVALID_ARGUMENT, "scale must be positive and finite");
+    if ((seqstart_q == nullptr) != (seqstart_k == nullptr)) return fail(FCK_ERR_INVALID_ARGUMENT, "group mode needs both seqstart_q and seqstart_k");
+    fck::PrefillArgs a{};
+    a.q = q;
+    a.k = k;
+    a.v = v;
+    a.o = o;
+    a.seqstart_q = seqstart_q;
+    a.batch = (int32_t)batch;
+    a.sq = (int32_t)seqlen_q;
+    a.hq = (int32_t)hq;
+    a.hk = (int32_t)hk;
+    a.scale_log2 = scale * fck::kLog2e;
+    a.mask_type = mask_type;
+    a.window_left = window_left;
+    a.window_right = window_right;
+    a.kv.page_shift = -1;
+    if (seqstart_q) {
+        a.kv.mode = 1;
+        a.kv.seqstart_k = seqstart_k;
+    } else {
+        if (seqlen_q <= 0 || seqlen_k <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch mode needs seqlen_q, seqlen_k > 0");
+        a.kv.mode = 0;
+        a.kv.seqlen_k = (int32_t)seqlen_k;
+        a.kv.seqlen_k_ptr = seqlen_k_ptr;
+        if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
+    }
+    return prefill_common(a, d, dtype, q_max_seq_len, true, stream, "FmhaFwd launch");
+}
+
+int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
+                           const int32_t* kv_indptr, const int32_t* kv_page_indices, const int32_t* kv_last_page_lens,
+                           int64_t num_total_pages, int64_t page_block_size, int64_t batch, int64_t hq, int64_t hk, int64_t d,
+                           int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left, int64_t window_right,
+                           uint32_t mask_type, int32_t dtype, void* stream)
+{
+    g_err[0] = 0;
+    if (int rc = check_common(batch, hq, hk, d, dv, dtype, nullptr)) return rc;
+    if (int rc = check_mask(mask_type)) return rc;
+    if (!q || !k_cache || !v_cache || !o || !seqstart_q || !kv_indptr || !kv_page_indices)
+        return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, seqstart_q, kv_indptr and kv_page_indices must not be null");
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache and o must be 16-byte aligned");
+    if (page_block_size <= 0 || num_total_pages <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "page_block_size and num_total_pages must be positive");
+    if (!(scale > 0.f) || !std::isfinite(scale)) return fail(FCK_ERR_INVALID_ARGUMENT, "scale must be positive and finite");
+    fck::PrefillArgs a{};
+    a.q = q;
+    a.k = k_cache;
+    a.v = v_cache;
+    a.o = o;
+    a.seqstart_q = seqstart_q;
+    a.batch = (int32_t)batch;
+    a.hq = (int32_t)hq;
+    a.hk = (int32_t)hk;
+    a.scale_log2 = scale * fck::kLog2e;
+    a.mask_type = mask_type;
+    a.window_left = window_left;
+    a.window_right = window_right;
+    a.kv.mode = 3;
+    a.kv.kv_indptr = kv_indptr;
+    a.kv.kv_page_indices = kv_page_indices;
+    a.kv.kv_last_page_lens = kv_last_page_lens;
+    a.kv.page_size = (int32_t)page_block_size;
+    a.kv.page_shift = log2_exact(page_block_size);
+    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdBatchPrefill launch");
+}
+
+int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
+                         const int32_t* seqlen_k_ptr, const int32_t* block_table, int64_t batch_stride_block_table,
+                         int64_t page_block_size, int64_t batch, int64_t seqlen_q, int64_t hq, int64_t hk, int64_t d,
+                         int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left, int64_t window_right,
+                         uint32_t mask_type, int32_t dtype, void* stream)
+{
+    g_err[0] = 0;
+    if (int rc = check_common(batch, hq, hk, d, dv, dtype, nullptr)) return rc;
+    if (int rc = check_mask(mask_type)) return rc;
+    if (!q || !k_cache || !v_cache || !o || !seqlen_k_ptr || !block_table)
+        return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, seqlen_k and block_table must not be null");
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache and o must be 16-byte aligned");
+    if (page_block_size <= 0 || batch_stride_block_table <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "page_block_size and batch_stride_block_table must be positive");
+    if (!(scale > 0.f) || !std::isfinite(scale)) return fail(FCK_ERR_INVALID_ARGUMENT, "scale must be positive and finite");
+    if (!seqstart_q && seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch mode needs seqlen_q > 0");
+    fck::PrefillArgs a{};
+    a.q = q;
+    a.k = k_cache;
+    a.v = v_cache;
+    a.o = o;
+    a.seqstart_q = seqstart_q;
+    a.batch = (int32_t)batch;
+    a.sq = (int32_t)seqlen_q;
+    a.hq = (int32_t)hq;
+    a.hk = (int32_t)hk;
+    a.scale_log2 = scale * fck::kLog2e;
+    a.mask_type = mask_type;
+    a.window_left = window_left;
+    a.window_right = window_right;
+    a.kv.mode = 2;
+    a.kv.block_table = block_table;
+    a.kv.block_table_stride = (int32_t)batch_stride_block_table;
+    a.kv.seqlen_k_ptr = seqlen_k_ptr;
+    a.kv.page_size = (int32_t)page_block_size;
+    a.kv.page_shift = log2_exact(page_block_size);
+    if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
+    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdPagedKV launch");
+}
+
+}  // extern "C"

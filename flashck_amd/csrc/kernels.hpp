@@ -1,0 +1,71 @@
+// Argument blocks and launchers shared between the C ABI (fmha_api.cpp) and the kernel translation units.
+#pragma once
+
+#include "common.hpp"
+
+namespace fck {
+
+struct SplitKvArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    float* o_acc;
+    float* lse_acc;
+    const int32_t* seqstart_q;
+    KvAddr kv;
+    int32_t batch, sq, hq, hk, num_splits;
+    int64_t shape_sq;  // Sq of the workspace: sq (batch mode) or total_q (group mode)
+    float scale_log2;  // scale * log2(e)
+    uint32_t mask_type;
+    int64_t window_left, window_right;
+};
+
+struct CombineArgs {
+    const float* lse_acc;
+    const float* o_acc;
+    void* o;
+    int64_t rows;  // Bs * Sq
+    int64_t Sq;
+    int32_t hq, dv, num_splits;
+};
+
+struct AppendKvArgs {
+    void* q;
+    void* k_cache;
+    void* v_cache;
+    const void* knew;
+    const void* vnew;
+    const int32_t* seqlen_k;
+    const int32_t* cu_seqlens_knew;
+    int32_t seqlen_knew;
+    const void* cos;
+    const void* sin;
+    int32_t rotary_dim, rope_mode, has_mask;
+    const int32_t* block_table;
+    int32_t block_table_stride, page_size;
+    const int32_t* cache_batch_idx;
+    int64_t seqlen_k_cache;
+    int32_t batch, hq, hk, d, dv;
+};
+
+struct PrefillArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    const int32_t* seqstart_q;
+    KvAddr kv;
+    int32_t batch, sq, hq, hk;
+    int32_t m_tiles;
+    float scale_log2;
+    uint32_t mask_type;
+    int64_t window_left, window_right;
+};
+
+hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page,
+                                 hipStream_t st);
+hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st);
+hipError_t launch_appendkv(const AppendKvArgs& a, int dtype, int max_new, hipStream_t st);
+hipError_t launch_prefill(const PrefillArgs& a, int d, int dtype, bool uniform_page, hipStream_t st);
+
+}  // namespace fck

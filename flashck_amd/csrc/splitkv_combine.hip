@@ -1,0 +1,70 @@
+// LSE combine of split-KV partial results (gfx950).
+//   LSE = logsumexp_s lse_acc[s];  O = sum_s exp(lse_acc[s] - LSE) * o_acc[s]  -> T
+// A pure streaming reduce: DV/4 lanes own one output row with float4 loads of each split's partial row.
+// Layouts: o_acc [Bs, Hq, ns, Sq, Dv], lse_acc [Bs, Hq, ns, Sq], o [Bs*Sq, Hq, Dv].
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace fck {
+
+template <typename T, int DV>
+__global__ __launch_bounds__(256) void splitkv_combine_kernel(const CombineArgs a)
+{
+    constexpr int TPR = DV / 4;     // threads per output row
+    constexpr int RPB = 256 / TPR;  // rows per block
+    const int64_t item = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;  // (row, head) pair
+    const int c = (threadIdx.x % TPR) * 4;
+    if (item >= a.rows * a.hq) return;
+    const int64_t row = item / a.hq;  // b * Sq + i
+    const int h = (int)(item % a.hq);
+    const int64_t b = row / a.Sq, i = row % a.Sq;
+    const int ns = a.num_splits;
+    const int64_t w0 = ((b * a.hq + h) * ns) * a.Sq + i;  // split 0; next split is Sq further
+
+    float m = -INFINITY;
+    for (int s = 0; s < ns; ++s) m = fmaxf(m, a.lse_acc[w0 + s * a.Sq]);
+    float sum = 0.f;
+    if (m != -INFINITY)
+        for (int s = 0; s < ns; ++s) sum += __expf(a.lse_acc[w0 + s * a.Sq] - m);
+    const float L = (sum == 0.f) ? -INFINITY : __logf(sum) + m;
+
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    if (L != -INFINITY)
+        for (int s = 0; s < ns; ++s) {
+            const float w = __expf(a.lse_acc[w0 + s * a.Sq] - L);
+            const f32x4_t v = *reinterpret_cast<const f32x4_t*>(a.o_acc + (w0 + s * a.Sq) * DV + c);
+            acc += w * v;
+        }
+    u32x2_t out;
+    out[0] = T::pack2(acc[0], acc[1]);
+    out[1] = T::pack2(acc[2], acc[3]);
+    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.o) + (row * a.hq + h) * DV + c) = out;
+}
+
+template <typename T, int DV>
+static hipError_t launch_dv(const CombineArgs& a, hipStream_t st)
+{
+    constexpr int RPB = 256 / (DV / 4);
+    const int64_t items = a.rows * a.hq;
+    const dim3 grid((unsigned)((items + RPB - 1) / RPB));
+    hipLaunchKernelGGL((splitkv_combine_kernel<T, DV>), grid, dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_t(const CombineArgs& a, hipStream_t st)
+{
+    switch (a.dv) {
+    case 64: return launch_dv<T, 64>(a, st);
+    case 128: return launch_dv<T, 128>(a, st);
+    case 256: return launch_dv<T, 256>(a, st);
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st)
+{
+    return dtype == 4 ? launch_t<BF16>(a, st) : launch_t<FP16>(a, st);
+}
+
+}  // namespace fck

@@ -1,0 +1,327 @@
+"""Functional FMHA operators: the `flash_ck.ops.fmha` surface FlashCK declares but leaves empty
+(flash_ck/utils/utils.py:49-58; tests/pytorch/fmha/test_{fmha_fwd,fmha_fwd_var_len,fmha_fwd_append_kv,
+batch_prefill}.py are 0-byte files), backed by the gfx950 kernels through the C ABI.
+
+The wrappers follow flash_ck/ops/norm/layer_norm.py:61-116 for validation (TypeError / ValueError before any
+launch).  Unlike that operator there is no PyTorch fallback: a missing library or a rejected call raises.
+
+Tensor conventions (T = torch.float16 | torch.bfloat16, contiguous, on the GPU):
+    q, o         [B, sq, Hq, D]  or packed [total_q, Hq, D] with cu_seqlens_q (int32 [B+1])
+    k, v         [B, sk, Hk, D]  or packed [total_k, Hk, D] with cu_seqlens_k
+    k/v_cache    paged [num_pages, page_size, Hk, D] with block_table int32 [B, max_pages_per_seq]
+    seqlen_k     int32 [B] valid keys per sequence
+"""
+import ctypes
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from ... import _lib
+from ...utils import FlashCKOperationType, register_flashck_functions
+
+__all__ = [
+    "MASK_NONE", "MASK_TOP_LEFT", "MASK_BOTTOM_RIGHT", "MASK_GENERIC", "ROPE_NONE", "ROPE_INTERLEAVED",
+    "ROPE_HALF_ROTATED", "fmha_fwd", "fmha_fwd_varlen", "fmha_fwd_splitkv", "fmha_fwd_splitkv_combine",
+    "fmha_fwd_appendkv", "fmha_batch_prefill", "fmha_fwd_pagedkv", "fmha_decode_paged", "num_splits_heuristic",
+    "splitkv_workspace",
+]
+
+# GenericAttentionMaskEnum / RopeEnum, core/profiling/attention/fmha_library.h:81-87,195-200
+MASK_NONE, MASK_TOP_LEFT, MASK_BOTTOM_RIGHT, MASK_GENERIC = 0, 1, 2, 3
+ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALF_ROTATED = 0, 1, 2
+
+_DTYPE_ID = {torch.float16: 3, torch.bfloat16: 4}  # flashck::DataType, core/utils/dtype.h:16-28
+
+
+def _dtype_id(t: torch.Tensor) -> int:
+    if t.dtype not in _DTYPE_ID:
+        raise TypeError(f"FMHA supports torch.float16 and torch.bfloat16, got {t.dtype}")
+    return _DTYPE_ID[t.dtype]
+
+
+def _check_tensor(name, t, dtype=None, ndim=None, optional=False):
+    if t is None:
+        if optional:
+            return
+        raise TypeError(f"{name} must be a torch.Tensor, got None")
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"Expected {name} to be a torch.Tensor, got {type(t)}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got device {t.device})")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must have dtype {dtype}, got {t.dtype}")
+    if ndim is not None and t.dim() not in (ndim if isinstance(ndim, tuple) else (ndim,)):
+        raise ValueError(f"{name} must have {ndim} dimensions, got shape {tuple(t.shape)}")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _call(name, *args):
+    lib = _lib.load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        msg = lib.fck_last_error().decode()
+        if rc == -2:
+            raise NotImplementedError(f"{name}: {msg}")
+        if rc == -1:
+            raise ValueError(f"{name}: {msg}")
+        raise RuntimeError(f"{name} failed ({rc}): {msg}")
+
+
+def _scale(scale, d):
+    # scale == 0 selects 1/sqrt(head_dim), as the FlashCK harness does (fmha_fwd_split_kv_jinja.h:60-62)
+    return float(scale) if scale else 1.0 / math.sqrt(d)
+
+
+def _window(window):
+    wl, wr = window
+    return int(wl), int(wr)
+
+
+def num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, num_cu=0) -> int:
+    """Split count chosen from the CU count and the KV length."""
+    return int(_lib.load().fck_fmha_num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k,
+                                                         head_dim, num_cu))
+
+
+def splitkv_workspace(shape_batch, q_num_heads, shape_seqlen_q, v_head_dim, num_splits, device) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(o_acc fp32 [Bs,Hq,ns,Sq,Dv], lse_acc fp32 [Bs,Hq,ns,Sq]) - fmha_fwd_split_kv_jinja.h:543-547."""
+    o_acc = torch.empty(shape_batch, q_num_heads, num_splits, shape_seqlen_q, v_head_dim, dtype=torch.float32, device=device)
+    lse_acc = torch.empty(shape_batch, q_num_heads, num_splits, shape_seqlen_q, dtype=torch.float32, device=device)
+    return o_acc, lse_acc
+
+
+def fmha_fwd(q, k, v, scale: float = 0.0, mask_type: int = MASK_NONE, window: Tuple[int, int] = (-1, -1),
+             seqlen_k: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Dense attention, batch mode: q [B,sq,Hq,D], k/v [B,sk,Hk,D] -> o [B,sq,Hq,D]."""
+    _check_tensor("q", q, ndim=4)
+    _check_tensor("k", k, dtype=q.dtype, ndim=4)
+    _check_tensor("v", v, dtype=q.dtype, ndim=4)
+    _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1, optional=True)
+    B, sq, Hq, D = q.shape
+    if k.shape[0] != B or v.shape[:3] != k.shape[:3]:
+        raise ValueError(f"k {tuple(k.shape)} / v {tuple(v.shape)} do not match q {tuple(q.shape)}")
+    if q.numel() == 0:
+        raise ValueError("Input tensor cannot be empty")
+    sk, Hk, Dv = k.shape[1], k.shape[2], v.shape[3]
+    o = out if out is not None else torch.empty(B, sq, Hq, Dv, dtype=q.dtype, device=q.device)
+    wl, wr = _window(window)
+    _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), None, None, _ptr(seqlen_k), B, sq, sk, Hq, Hk, D, Dv,
+          sq, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    return o
+
+
+def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scale: float = 0.0,
+                    mask_type: int = MASK_NONE, window=(-1, -1), out=None) -> torch.Tensor:
+    """Dense attention, group mode: q [total_q,Hq,D], k/v [total_k,Hk,D] packed by cu_seqlens."""
+    _check_tensor("q", q, ndim=3)
+    _check_tensor("k", k, dtype=q.dtype, ndim=3)
+    _check_tensor("v", v, dtype=q.dtype, ndim=3)
+    _check_tensor("cu_seqlens_q", cu_seqlens_q, dtype=torch.int32, ndim=1)
+    _check_tensor("cu_seqlens_k", cu_seqlens_k, dtype=torch.int32, ndim=1)
+    if cu_seqlens_q.numel() != cu_seqlens_k.numel() or cu_seqlens_q.numel() < 2:
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must both have batch + 1 entries")
+    B = cu_seqlens_q.numel() - 1
+    tq, Hq, D = q.shape
+    Hk, Dv = k.shape[1], v.shape[2]
+    o = out if out is not None else torch.empty(tq, Hq, Dv, dtype=q.dtype, device=q.device)
+    wl, wr = _window(window)
+    _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), None, B, tq,
+          k.shape[0], Hq, Hk, D, Dv, max_seqlen_q, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    return o
+
+
+def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=None, cache_batch_idx=None,
+                     cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q: int = 0, scale: float = 0.0,
+                     mask_type: int = MASK_NONE, window=(-1, -1), o_acc=None, lse_acc=None):
+    """Split-KV forward: returns the per-split partials (o_acc, lse_acc), to be merged by fmha_fwd_splitkv_combine.
+
+    k/v are a paged cache when block_table is given, packed when cu_seqlens_k is given, else [B*, sk, Hk, D].
+    """
+    group = cu_seqlens_q is not None
+    _check_tensor("q", q, ndim=3 if group else 4)
+    _check_tensor("k", k, dtype=q.dtype)
+    _check_tensor("v", v, dtype=q.dtype)
+    for name, t in (("seqlen_k", seqlen_k), ("block_table", block_table), ("cache_batch_idx", cache_batch_idx),
+                    ("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
+        _check_tensor(name, t, dtype=torch.int32, optional=True)
+    if int(num_splits) < 1:
+        raise ValueError("num_splits must be >= 1")
+    Hq, D = q.shape[-2], q.shape[-1]
+    Hk, Dv = k.shape[-2], v.shape[-1]
+    if group:
+        B, sq, bs = cu_seqlens_q.numel() - 1, q.shape[0], 1
+        if max_seqlen_q <= 0:
+            raise ValueError("group mode needs max_seqlen_q")
+    else:
+        B, sq, bs = q.shape[0], q.shape[1], q.shape[0]
+        max_seqlen_q = sq
+    if block_table is not None:
+        if seqlen_k is None:
+            raise ValueError("a paged cache needs seqlen_k")
+        if block_table.dim() != 2 or block_table.shape[0] != B:
+            raise ValueError(f"block_table must be [batch, max_pages_per_seq], got {tuple(block_table.shape)}")
+        page, sk, max_blocks = k.shape[1], 0, block_table.numel()
+    else:
+        page, max_blocks = 0, 0
+        sk = k.shape[0] if cu_seqlens_k is not None else k.shape[1]
+    if o_acc is None or lse_acc is None:
+        o_acc, lse_acc = splitkv_workspace(bs, Hq, sq, Dv, num_splits, q.device)
+    wl, wr = _window(window)
+    _call("fck_fmha_fwd_splitkv", _ptr(q), _ptr(k), _ptr(v), None, _ptr(lse_acc), _ptr(o_acc), _ptr(cu_seqlens_q),
+          _ptr(cu_seqlens_k), _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv,
+          max_seqlen_q, int(num_splits), max_blocks, page, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    return o_acc, lse_acc
+
+
+def fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype, cu_seqlens_q=None, max_seqlen_q: int = 0, out=None) -> torch.Tensor:
+    """LSE combine of split-KV partials -> o [B,sq,Hq,Dv] (or [total_q,Hq,Dv] in group mode)."""
+    _check_tensor("lse_acc", lse_acc, dtype=torch.float32, ndim=4)
+    _check_tensor("o_acc", o_acc, dtype=torch.float32, ndim=5)
+    _check_tensor("cu_seqlens_q", cu_seqlens_q, dtype=torch.int32, optional=True)
+    if dtype not in _DTYPE_ID:
+        raise TypeError(f"FMHA supports torch.float16 and torch.bfloat16, got {dtype}")
+    bs, Hq, ns, sq, Dv = o_acc.shape
+    if tuple(lse_acc.shape) != (bs, Hq, ns, sq):
+        raise ValueError(f"lse_acc {tuple(lse_acc.shape)} does not match o_acc {tuple(o_acc.shape)}")
+    if cu_seqlens_q is not None:
+        B = cu_seqlens_q.numel() - 1
+        o = out if out is not None else torch.empty(sq, Hq, Dv, dtype=dtype, device=o_acc.device)
+    else:
+        B = bs
+        o = out if out is not None else torch.empty(bs, sq, Hq, Dv, dtype=dtype, device=o_acc.device)
+    _call("fck_fmha_fwd_splitkv_combine", _ptr(lse_acc), _ptr(o_acc), _ptr(o), _ptr(cu_seqlens_q), B, sq, Hq, Dv,
+          max_seqlen_q or sq, ns, _DTYPE_ID[dtype], _stream())
+    return o
+
+
+def fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, *, cu_seqlens_knew=None, max_seqlen_knew: int = 0,
+                      rotary_cos=None, rotary_sin=None, rope_mode: int = ROPE_NONE, has_mask: bool = True,
+                      block_table=None, cache_batch_idx=None) -> None:
+    """Rotate knew (and q, in place) and append knew/vnew to the cache behind seqlen_k[b] tokens; in place.
+
+    knew/vnew/q are packed [total_new, H, D] with cu_seqlens_knew, or [B, n, H, D] with n new tokens everywhere.
+    seqlen_k is NOT advanced: the caller adds the new counts, as with the ck_tile kernel.
+    """
+    packed = cu_seqlens_knew is not None
+    _check_tensor("knew", knew, ndim=3 if packed else 4)
+    _check_tensor("vnew", vnew, dtype=knew.dtype, ndim=3 if packed else 4)
+    _check_tensor("q", q, dtype=knew.dtype, ndim=3 if packed else 4, optional=True)
+    _check_tensor("k_cache", k_cache, dtype=knew.dtype, ndim=4)
+    _check_tensor("v_cache", v_cache, dtype=knew.dtype, ndim=4)
+    _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1)
+    for name, t in (("cu_seqlens_knew", cu_seqlens_knew), ("block_table", block_table), ("cache_batch_idx", cache_batch_idx)):
+        _check_tensor(name, t, dtype=torch.int32, optional=True)
+    _check_tensor("rotary_cos", rotary_cos, dtype=knew.dtype, ndim=2, optional=True)
+    _check_tensor("rotary_sin", rotary_sin, dtype=knew.dtype, ndim=2, optional=True)
+    B = seqlen_k.numel()
+    Hk, D, Dv = knew.shape[-2], knew.shape[-1], vnew.shape[-1]
+    Hq = q.shape[-2] if q is not None else 0
+    if packed:
+        if max_seqlen_knew <= 0:
+            raise ValueError("packed new tokens need max_seqlen_knew")
+        n = max_seqlen_knew
+    else:
+        n = knew.shape[1]
+    if rope_mode != ROPE_NONE:
+        if rotary_cos is None or rotary_sin is None:
+            raise ValueError("rope_mode != ROPE_NONE needs rotary_cos and rotary_sin")
+        rotary_dim = rotary_cos.shape[1] * 2
+    else:
+        rotary_dim = 0
+    if block_table is not None:
+        stride, page, rows = block_table.shape[1], k_cache.shape[1], 0
+    else:
+        stride, page, rows = 0, 0, k_cache.shape[1]
+    _call("fck_fmha_fwd_appendkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(knew), _ptr(vnew), _ptr(seqlen_k),
+          _ptr(cu_seqlens_knew), n, _ptr(rotary_cos), _ptr(rotary_sin), rotary_dim, rope_mode, int(bool(has_mask)),
+          _ptr(block_table), stride, page, _ptr(cache_batch_idx), rows, B, Hq, Hk, D, Dv, _dtype_id(knew), _stream())
+
+
+def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_indices, kv_last_page_lens=None, *,
+                       max_seqlen_q: int, scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0),
+                       out=None) -> torch.Tensor:
+    """Varlen prefill over a page list: q [total_q,Hq,D]; sequence b owns pages
+    kv_page_indices[kv_indptr[b]:kv_indptr[b+1]] of the cache [num_pages, page_size, Hk, D]."""
+    _check_tensor("q", q, ndim=3)
+    _check_tensor("k_cache", k_cache, dtype=q.dtype, ndim=4)
+    _check_tensor("v_cache", v_cache, dtype=q.dtype, ndim=4)
+    for name, t in (("cu_seqlens_q", cu_seqlens_q), ("kv_indptr", kv_indptr), ("kv_page_indices", kv_page_indices)):
+        _check_tensor(name, t, dtype=torch.int32, ndim=1)
+    _check_tensor("kv_last_page_lens", kv_last_page_lens, dtype=torch.int32, ndim=1, optional=True)
+    B = cu_seqlens_q.numel() - 1
+    if kv_indptr.numel() != B + 1:
+        raise ValueError("kv_indptr must have batch + 1 entries")
+    tq, Hq, D = q.shape
+    num_pages, page, Hk, Dv = v_cache.shape
+    o = out if out is not None else torch.empty(tq, Hq, Dv, dtype=q.dtype, device=q.device)
+    wl, wr = _window(window)
+    _call("fck_fmha_batch_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
+          _ptr(kv_page_indices), _ptr(kv_last_page_lens), num_pages, page, B, Hq, Hk, D, Dv, max_seqlen_q,
+          _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    return o
+
+
+def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q=None, max_seqlen_q: int = 0,
+                     scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0), out=None) -> torch.Tensor:
+    """Prefill over a block table (no splits): q [B,sq,Hq,D] or packed [total_q,Hq,D]."""
+    group = cu_seqlens_q is not None
+    _check_tensor("q", q, ndim=3 if group else 4)
+    _check_tensor("k_cache", k_cache, dtype=q.dtype, ndim=4)
+    _check_tensor("v_cache", v_cache, dtype=q.dtype, ndim=4)
+    _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1)
+    _check_tensor("block_table", block_table, dtype=torch.int32, ndim=2)
+    _check_tensor("cu_seqlens_q", cu_seqlens_q, dtype=torch.int32, ndim=1, optional=True)
+    B = seqlen_k.numel()
+    Hq, D = q.shape[-2], q.shape[-1]
+    _, page, Hk, Dv = v_cache.shape
+    sq = 0 if group else q.shape[1]
+    if group and max_seqlen_q <= 0:
+        raise ValueError("group mode needs max_seqlen_q")
+    o = out if out is not None else torch.empty(*q.shape[:-1], Dv, dtype=q.dtype, device=q.device)
+    wl, wr = _window(window)
+    _call("fck_fmha_fwd_pagedkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
+          _ptr(block_table), block_table.shape[1], page, B, sq, Hq, Hk, D, Dv, max_seqlen_q or sq, _scale(scale, D), wl, wr,
+          mask_type, _dtype_id(q), _stream())
+    return o
+
+
+def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits: int = 0, max_seqlen_k: int = 0,
+                      cu_seqlens_q=None, max_seqlen_q: int = 0, scale: float = 0.0, mask_type: int = MASK_NONE,
+                      window=(-1, -1), workspace=None, out=None) -> torch.Tensor:
+    """Paged decode = split-KV forward + LSE combine; num_splits = 0 asks the heuristic (needs max_seqlen_k)."""
+    group = cu_seqlens_q is not None
+    Hq, D = q.shape[-2], q.shape[-1]
+    Hk = k_cache.shape[2]
+    B = seqlen_k.numel()
+    sq = max_seqlen_q if group else q.shape[1]
+    if num_splits <= 0:
+        if max_seqlen_k <= 0:
+            max_seqlen_k = block_table.shape[1] * k_cache.shape[1]
+        num_splits = num_splits_heuristic(B, Hq, Hk, sq, max_seqlen_k, D)
+    o_acc, lse_acc = workspace if workspace is not None else (None, None)
+    o_acc, lse_acc = fmha_fwd_splitkv(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_k, block_table=block_table,
+                                      cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, scale=scale,
+                                      mask_type=mask_type, window=window, o_acc=o_acc, lse_acc=lse_acc)
+    return fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, out=out)
+
+
+register_flashck_functions(FlashCKOperationType.FMHA.value, {
+    "forward": fmha_fwd,
+    "forward_varlen": fmha_fwd_varlen,
+    "forward_splitkv": fmha_fwd_splitkv,
+    "forward_splitkv_combine": fmha_fwd_splitkv_combine,
+    "forward_appendkv": fmha_fwd_appendkv,
+    "batch_prefill": fmha_batch_prefill,
+    "forward_pagedkv": fmha_fwd_pagedkv,
+    "decode_paged": fmha_decode_paged,
+})

@@ -1,0 +1,173 @@
+/*
+ * C ABI of the MI355X (gfx950) FMHA forward library: split-KV forward + LSE combine, appendKV (rotary embedding +
+ * paged-cache write), paged-KV attention and varlen batch prefill.
+ *
+ * Each entry point keeps the parameter order of the generated-library function FlashCK would dlsym for the same
+ * operation (paths relative to the FlashCK tree), made C-clean:
+ *   - `int` status instead of `void` + a message on std::cerr (fmha_common_jinja.h:5-12,58-60);
+ *     0 = success, negative = FCK_ERR_*; fck_last_error() holds the text for the calling thread;
+ *   - index arrays are int32 (FlashCK declares int64_t*, but the ck_tile kernels it instantiates read int32:
+ *     ck_tile/ops/fmha/kernel/fmha_fwd_splitkv_kernel.hpp:263-264,491-492);
+ *   - `std::array<int64_t,2> window_size` becomes two int64_t;
+ *   - an explicit `dtype` (flashck::DataType id, core/utils/dtype.h:16-28) replaces the per-type instantiation.
+ *
+ * Conventions: every pointer is caller-owned device memory (workspaces included); launches are asynchronous on
+ * `stream` (a hipStream_t passed as void*), nothing synchronises; no entry point allocates; the library keeps no
+ * mutable state except the calling thread's last error text, so calls are re-entrant and stream-ordered.
+ *
+ * Tensor layouts (element strides; T = fp16 or bf16, 2 bytes):
+ *   Q, O        batch mode [B, sq, Hq, D|Dv]; group mode (seqstart_q != NULL) [total_q, Hq, D|Dv]
+ *   K, V        batch [B, sk, Hk, D|Dv]; group [total_k, Hk, D|Dv]; paged [num_pages, P, Hk, D|Dv]
+ *               (fmha_fwd_split_kv_jinja.h:261-263,277-279,294-306,511-522)
+ *   block_table int32 [B, max_num_page_blocks / B]        (fmha_fwd_split_kv_jinja.h:318,549-552)
+ *   o_acc       fp32  [Bs, Hq, num_splits, Sq, Dv]        (fmha_fwd_split_kv_jinja.h:289,308,323,546-547)
+ *   lse_acc     fp32  [Bs, Hq, num_splits, Sq]            (fmha_fwd_split_kv_combine_jinja.h:129,134,139)
+ *               with (Bs, Sq) = (B, sq) in batch mode and (1, total_q) in group mode
+ */
+#ifndef FLASHCK_FMHA_C_API_H
+#define FLASHCK_FMHA_C_API_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FCK_EXPORT __attribute__((visibility("default")))
+
+/* flashck::DataType, core/utils/dtype.h:16-28 */
+#define FCK_DTYPE_FP16 3
+#define FCK_DTYPE_BF16 4
+
+/* GenericAttentionMaskEnum, core/profiling/attention/fmha_library.h:81-87 */
+#define FCK_MASK_NONE 0
+#define FCK_MASK_TOP_LEFT 1
+#define FCK_MASK_BOTTOM_RIGHT 2
+#define FCK_MASK_GENERIC 3
+
+/* RopeEnum, core/profiling/attention/fmha_library.h:195-200 */
+#define FCK_ROPE_NONE 0
+#define FCK_ROPE_INTERLEAVED 1
+#define FCK_ROPE_HALF_ROTATED 2
+
+#define FCK_OK 0
+#define FCK_ERR_INVALID_ARGUMENT (-1) /* null pointer, non-positive size, Hq % Hk != 0 ... */
+#define FCK_ERR_UNSUPPORTED (-2)      /* dtype / head_dim / feature this build has no kernel for */
+#define FCK_ERR_LAUNCH (-3)           /* the HIP runtime refused the launch */
+
+/* Text of the last error raised on the calling thread ("" when none). */
+FCK_EXPORT const char* fck_last_error(void);
+
+/* Library version string. */
+FCK_EXPORT const char* fck_fmha_version(void);
+
+/*
+ * Dense / varlen forward.  Replaces `FmhaFwd`, fmha_fwd/fmha_fwd_jinja.h:124-147 (args :68-122, strides :186-304).
+ * batch mode: seqstart_q = seqstart_k = NULL; seqlen_k_ptr optional per-batch key counts.
+ * group mode: seqstart_q / seqstart_k are int32 [B+1] prefix sums; seqlen_q / seqlen_k are ignored.
+ */
+FCK_EXPORT int fck_fmha_fwd(const void* q, const void* k, const void* v, const void* bias, void* o,
+                            const int32_t* seqstart_q, const int32_t* seqstart_k, const int32_t* seqlen_k_ptr,
+                            int64_t batch, int64_t seqlen_q, int64_t seqlen_k, int64_t q_num_heads,
+                            int64_t kv_num_heads, int64_t qk_head_dim, int64_t v_head_dim, int64_t q_max_seq_len,
+                            float scale, int64_t window_left, int64_t window_right, uint32_t mask_type,
+                            int32_t dtype, void* stream);
+
+/*
+ * Split-KV forward: per split s of num_splits, attention over keys [s*ceil(Lk/ns), min(Lk,(s+1)*ceil(Lk/ns)))
+ * written as per-split normalised fp32 o_acc and lse_acc (= max + ln(sum), -inf for a split with no visible key).
+ * Replaces `FmhaFwdSplitKV`, fmha_fwd_split_kv/fmha_fwd_split_kv_jinja.h:155-184 (args :76-151, strides :241-409).
+ * K/V addressing: block_table != NULL -> paged cache with page_block_size tokens per page and per-sequence key
+ * counts in seqlen_k_ptr; else seqstart_k != NULL -> group mode; else batch cache [*, seqlen_k, Hk, D] whose row
+ * is cache_batch_idx[b] when that is given, with key counts seqlen_k_ptr[b] (or seqlen_k when NULL).
+ */
+FCK_EXPORT int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v, const void* bias, void* lse_acc,
+                                    void* o_acc, const int32_t* seqstart_q, const int32_t* seqstart_k,
+                                    const int32_t* seqlen_k_ptr, const int32_t* block_table,
+                                    const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
+                                    int64_t seqlen_k, int64_t q_num_heads, int64_t kv_num_heads, int64_t qk_head_dim,
+                                    int64_t v_head_dim, int64_t q_max_seq_len, int64_t num_splits,
+                                    int64_t max_num_page_blocks, int64_t page_block_size, float scale,
+                                    int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype,
+                                    void* stream);
+
+/*
+ * LSE combine: O = sum_s exp(lse_acc[s] - logsumexp_s lse_acc) * o_acc[s], stored as T.
+ * Replaces `FmhaSplitKVCombine` / `FmhaFwdSplitKVCombine`, fmha_fwd_split_kv_combine_jinja.h:78-92
+ * (args :37-76, strides :114-165), declared at fmha_fwd_split_kv_combine_call.h:26-36.
+ * seqstart_q != NULL selects group mode (seqlen_q is then ignored; rows = seqstart_q[B]).
+ */
+FCK_EXPORT int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o,
+                                            const int32_t* seqstart_q, int64_t batch, int64_t seqlen_q,
+                                            int64_t q_num_heads, int64_t v_head_dim, int64_t q_max_seq_len,
+                                            int64_t num_splits, int32_t dtype, void* stream);
+
+/*
+ * AppendKV: rotate knew (and q, in place) and write knew / vnew behind the seqlen_k[b] tokens each sequence
+ * already holds.  FlashCK only names this operation (FmhaKind::FwdAppendKV, fmha_library.h:19,41; config struct
+ * core/utils/json_config.h:280-312); the argument list follows the ck_tile kernel it would instantiate
+ * (ck_tile/ops/fmha/kernel/fmha_fwd_appendkv_kernel.hpp:146-231).
+ *   q      [total_new, Hq, D] (cu_seqlens_knew given) or [B, seqlen_knew, Hq, D]; may be NULL
+ *   knew   [total_new, Hk, D] or [B, seqlen_knew, Hk, D];  vnew likewise with Dv
+ *   cu_seqlens_knew  int32 [B+1] or NULL (then every sequence appends seqlen_knew tokens, the ck_tile form)
+ *   rotary_cos/sin   T [>= max position + 1, rotary_dim / 2]; row = absolute position
+ *   has_mask         query i uses position seqlen_k[b] + i when non-zero, seqlen_k[b] otherwise
+ *   block_table != NULL: paged cache; else batch cache with `seqlen_k_cache` rows per sequence, row chosen by
+ *   cache_batch_idx[b] when given.
+ */
+FCK_EXPORT int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* knew, const void* vnew,
+                                     const int32_t* seqlen_k, const int32_t* cu_seqlens_knew, int64_t seqlen_knew,
+                                     const void* rotary_cos, const void* rotary_sin, int64_t rotary_dim,
+                                     int32_t rope_mode, int32_t has_mask, const int32_t* block_table,
+                                     int64_t batch_stride_block_table, int64_t page_block_size,
+                                     const int32_t* cache_batch_idx, int64_t seqlen_k_cache, int64_t batch,
+                                     int64_t q_num_heads, int64_t kv_num_heads, int64_t qk_head_dim,
+                                     int64_t v_head_dim, int32_t dtype, void* stream);
+
+/*
+ * Varlen batch prefill over a page list.  FlashCK's problem definition:
+ * core/profiling/attention/fmha_fwd_batch_prefill/fmha_fwd_batch_prefill_problem.h:35-100 (kv_indptr,
+ * kv_page_indices, num_total_pages :98-99); kernel glue files are empty there.
+ *   q, o  [total_q, Hq, D|Dv] packed by seqstart_q (int32 [B+1])
+ *   sequence b owns pages kv_page_indices[kv_indptr[b] .. kv_indptr[b+1]) and
+ *   (n_pages - 1) * page_block_size + kv_last_page_lens[b] keys (full last page when kv_last_page_lens is NULL).
+ */
+FCK_EXPORT int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cache, void* o,
+                                      const int32_t* seqstart_q, const int32_t* kv_indptr,
+                                      const int32_t* kv_page_indices, const int32_t* kv_last_page_lens,
+                                      int64_t num_total_pages, int64_t page_block_size, int64_t batch,
+                                      int64_t q_num_heads, int64_t kv_num_heads, int64_t qk_head_dim,
+                                      int64_t v_head_dim, int64_t q_max_seq_len, float scale, int64_t window_left,
+                                      int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream);
+
+/*
+ * Prefill over a vLLM-style block table (no splits).  FlashCK's problem definition:
+ * core/profiling/attention/fmha_fwd_paged_kv_prefill/fmha_fwd_paged_kv_prefill_problem.h:35-97.
+ * seqstart_q NULL -> batch mode q [B, seqlen_q, Hq, D].
+ */
+FCK_EXPORT int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache, void* o,
+                                    const int32_t* seqstart_q, const int32_t* seqlen_k_ptr,
+                                    const int32_t* block_table, int64_t batch_stride_block_table,
+                                    int64_t page_block_size, int64_t batch, int64_t seqlen_q, int64_t q_num_heads,
+                                    int64_t kv_num_heads, int64_t qk_head_dim, int64_t v_head_dim,
+                                    int64_t q_max_seq_len, float scale, int64_t window_left, int64_t window_right,
+                                    uint32_t mask_type, int32_t dtype, void* stream);
+
+/*
+ * Split count from the CU count and the KV length.  FlashCK's command line promises "0 = heuristic"
+ * (fmha_fwd_split_kv_jinja.h:28-30) without implementing one; num_cu <= 0 asks the current device.
+ * Returns a value in [1, 128].
+ */
+FCK_EXPORT int fck_fmha_num_splits_heuristic(int64_t batch, int64_t q_num_heads, int64_t kv_num_heads,
+                                             int64_t seqlen_q, int64_t max_seqlen_k, int64_t head_dim,
+                                             int64_t num_cu);
+
+/* Bytes of o_acc followed by lse_acc for the shapes above (fmha_fwd_split_kv_jinja.h:543-547). */
+FCK_EXPORT size_t fck_fmha_splitkv_workspace_bytes(int64_t shape_batch, int64_t q_num_heads, int64_t shape_seqlen_q,
+                                                   int64_t v_head_dim, int64_t num_splits);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,30 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def orc():
+    from oracle import fmha_oracle
+    fmha_oracle.build()
+    return fmha_oracle
+
+
+@pytest.fixture(scope="session")
+def fmha():
+    """The HIP operators; a GPU test that gets here without the built library must fail, not skip."""
+    import torch
+    from flashck_amd import _lib
+    from flashck_amd.ops import fmha as ops
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    _lib.load()
+    return ops
