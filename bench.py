@@ -1,0 +1,222 @@
+#!/usr/bin/env python3
+"""Benchmark of the FMHA hot path on one MI355X.
+
+One "step" is one pass of the headline workload: split-KV long-context decode (batch 4, q_len 1, 64 query / 8 KV heads,
+head_dim 128, 32768 keys per sequence in shuffled 128-token pages, num_splits 8) = one split-KV launch + one combine
+launch.  `value` is algorithmic HBM bytes per step / wall time per step with every input resident in HBM; the KV pool is
+rotated over several copies so no step finds its pages in the caches.  The JSON line also carries the roofline of the
+dominant kernel (HIP events around every split-KV launch of the timed region), a CPU baseline (the oracle on a bounded
+sample, same run, host cores of this box) and, under "extra", the other workloads: paged decode, appendKV, and varlen
+causal prefill in TFLOP/s.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="splitkv", choices=["splitkv", "paged_decode", "prefill", "prefill256"],
+                    help="workload of the headline line (default: split-KV long-context decode)")
+    ap.add_argument("--copies", type=int, default=4, help="KV pool copies rotated between steps")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    return ap.parse_args()
+
+
+def time_steps(fn, steps, warmup, torch, kernel_events=False):
+    """Runs fn(step, ev) warmup + steps times; returns (wall seconds for `steps`, avg ms between event pairs)."""
+    for i in range(warmup):
+        fn(i, None)
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)] \
+        if kernel_events else [None] * steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(warmup + i, evs[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern_ms = None
+    if kernel_events:
+        kern_ms = sum(a.elapsed_time(b) for a, b in evs) / steps
+    return wall, kern_ms
+
+
+def bench_decode(args, torch, fmha, gen, which):
+    if which == "splitkv":
+        w = gen.workload_splitkv_decode()
+        ns = w["num_splits"]
+        name = "split-KV long-context decode: B=4 q=1 Hq64/Hk8 D128 L=32768 P=128 ns=8 + combine (bf16)"
+    else:
+        w = gen.workload_paged_decode()
+        ns = fmha.num_splits_heuristic(32, 32, 8, 1, max(w["lens"]), 128)
+        name = f"paged-KV decode: B=32 q=1 Hq32/Hk8 D128 L~U[512,4096] P=128 ns={ns} + combine (bf16)"
+    B, _, Hq, D = w["q"].shape
+    Hk = w["k_cache"].shape[2]
+    dev = "cuda"
+    q = w["q"].to(dev)
+    bt, sl = w["block_table"].to(dev), w["seqlen_k"].to(dev)
+    pools = [(w["k_cache"].to(dev), w["v_cache"].to(dev))]
+    for _ in range(args.copies - 1):
+        pools.append((pools[0][0].clone(), pools[0][1].clone()))
+    o_acc, lse_acc = fmha.splitkv_workspace(B, Hq, 1, D, ns, dev)
+    o = torch.empty(B, 1, Hq, D, dtype=q.dtype, device=dev)
+
+    def step(i, ev):
+        kc, vc = pools[i % len(pools)]
+        if ev is not None:
+            ev[0].record()
+        fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc)
+        if ev is not None:
+            ev[1].record()
+        fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, out=o)
+
+    wall, kern_ms = time_steps(step, args.steps, args.warmup, torch, kernel_events=True)
+    nbytes = gen.decode_bytes(w["lens"], [1] * B, Hq, Hk, D, D, 128)
+    flops = gen.decode_flops(w["lens"], [1] * B, Hq, D, D)
+    ms = wall / args.steps * 1e3
+    res = dict(name=name, ms_per_step=ms, bytes=nbytes, flops=flops, gbs=nbytes / (ms * 1e-3) / 1e9,
+               kernel_ms=kern_ms, kernel_gbs=nbytes / (kern_ms * 1e-3) / 1e9, num_splits=ns, w=w)
+    return res
+
+
+def bench_prefill(args, torch, fmha, gen, d, steps, warmup):
+    w = gen.workload_varlen_prefill(head_dim=d)
+    dev = "cuda"
+    a = [w[k].to(dev) for k in ("q", "k_cache", "v_cache", "cu_seqlens_q", "kv_indptr", "kv_page_indices", "kv_last_page_lens")]
+    o = torch.empty_like(a[0])
+
+    def step(i, ev):
+        if ev is not None:
+            ev[0].record()
+        fmha.fmha_batch_prefill(*a, max_seqlen_q=w["max_seqlen_q"], scale=w["scale"], out=o)
+        if ev is not None:
+            ev[1].record()
+
+    wall, kern_ms = time_steps(step, steps, warmup, torch, kernel_events=True)
+    flops = gen.prefill_flops(w["lens"], 32, d, d)
+    nbytes = gen.prefill_bytes(w["lens"], 32, 8, d, d)
+    ms = wall / steps * 1e3
+    return dict(name=f"varlen causal batch prefill: 16 seqs L~U[128,8192] Hq32/Hk8 D{d} paged P=128 (bf16)",
+                ms_per_step=ms, flops=flops, bytes=nbytes, tflops=flops / (ms * 1e-3) / 1e12, kernel_ms=kern_ms,
+                kernel_tflops=flops / (kern_ms * 1e-3) / 1e12, total_q=sum(w["lens"]))
+
+
+def bench_appendkv(args, torch, fmha, gen, steps, warmup):
+    w = gen.workload_appendkv_decode()
+    dev = "cuda"
+    q, kc, vc = w["q"].to(dev), w["k_cache"].to(dev), w["v_cache"].to(dev)
+    knew, vnew, sl, cu = w["knew"].to(dev), w["vnew"].to(dev), w["seqlen_k"].to(dev), w["cu_seqlens_knew"].to(dev)
+    cos, sin, bt = w["rotary_cos"].to(dev), w["rotary_sin"].to(dev), w["block_table"].to(dev)
+
+    def step(i, ev):
+        fmha.fmha_fwd_appendkv(q, kc, vc, knew, vnew, sl, cu_seqlens_knew=cu, max_seqlen_knew=w["max_new"], rotary_cos=cos,
+                               rotary_sin=sin, rope_mode=fmha.ROPE_HALF_ROTATED, has_mask=True, block_table=bt)
+
+    wall, _ = time_steps(step, steps, warmup, torch)
+    tn = q.shape[0]
+    nbytes = tn * (8 * 128 * 2 * 2) * 2 + tn * 32 * 128 * 2 * 2
+    return dict(name="appendKV + RoPE: B=16, 1-16 new tokens, Hq32/Hk8 D128, shuffled 128-token pages (bf16)",
+                us_per_call=wall / steps * 1e6, bytes=nbytes, new_tokens=tn)
+
+
+def cpu_baseline_decode(w, ns, gen, min_seconds=10.0):
+    """The oracle (a port of the reference's CPU host-reference attention) on the same workload: split-KV partials +
+    combine over every sequence and head, repeated until at least `min_seconds` of CPU work have been timed."""
+    from oracle import fmha_oracle as orc
+    orc.build()
+    q, bt, sl, lens = w["q"], w["block_table"], w["seqlen_k"], w["lens"]
+    B, Hq, D, Hk = q.shape[0], q.shape[2], q.shape[3], w["k_cache"].shape[2]
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        o_acc, lse_acc = orc.fmha_splitkv(q, w["k_cache"], w["v_cache"], ns, seqlen_k=sl, block_table=bt, scale=w["scale"])
+        orc.splitkv_combine(lse_acc, o_acc, q.dtype)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds or passes >= 1000:
+            break
+    nbytes = gen.decode_bytes(lens, [1] * B, Hq, Hk, D, D, 128) * passes
+    return dict(value=nbytes / dt / 1e9, unit="GB/s", cores=orc.num_threads(), kind="port",
+                sample=f"{passes} passes over the whole workload ({B} sequences, {Hq} heads, full KV lengths), "
+                       f"split-KV partials + combine, {dt:.1f} s of CPU time on {orc.num_threads()} threads",
+                seconds=dt, us_per_call=dt / passes * 1e6)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build has no multi-GPU path (asked for --gpus {args.gpus})", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    from flashck_amd import _lib, generators as gen
+    from flashck_amd.ops import fmha
+    _lib.load()  # raises when the HIP library is missing: there is no other compute path
+    torch.cuda.set_device(0)
+
+    extra = {}
+    if args.workload in ("splitkv", "paged_decode"):
+        r = bench_decode(args, torch, fmha, gen, args.workload)
+        value, unit, metric = r["gbs"], "GB/s", "paged-KV decode HBM GB/s (% of peak) + us/call; prefill TFLOP/s, MFMA util %"
+        roof = dict(bound="hbm", kernel="splitkv_decode_kernel", achieved=r["kernel_gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=r["kernel_gbs"] / HBM_PEAK_GBS, traffic=None, bytes_per_launch=r["bytes"],
+                    avg_launch_us=r["kernel_ms"] * 1e3)
+        extra["pct_of_hbm_peak"] = 100.0 * value / HBM_PEAK_GBS
+        extra["us_per_call"] = r["ms_per_step"] * 1e3
+        cpu = None
+        if not args.no_cpu:
+            cpu = cpu_baseline_decode(r["w"], r["num_splits"], gen)
+        ms, name = r["ms_per_step"], r["name"]
+    else:
+        d = 128 if args.workload == "prefill" else 256
+        r = bench_prefill(args, torch, fmha, gen, d, args.steps, args.warmup)
+        value, unit, metric = r["tflops"], "TFLOP/s", "varlen causal prefill TFLOP/s (MFMA util %)"
+        roof = dict(bound="mfma", kernel="prefill_kernel", achieved=r["kernel_tflops"], peak=MFMA_BF16_PEAK_TFLOPS,
+                    unit="TFLOP/s", frac=r["kernel_tflops"] / MFMA_BF16_PEAK_TFLOPS, traffic=None,
+                    flops_per_launch=r["flops"], avg_launch_us=r["kernel_ms"] * 1e3)
+        cpu = None
+        ms, name = r["ms_per_step"], r["name"]
+
+    if not args.no_extra and args.workload == "splitkv":
+        a2 = argparse.Namespace(**vars(args))
+        a2.steps, a2.warmup = max(20, args.steps // 2), 10
+        r2 = bench_decode(a2, torch, fmha, gen, "paged_decode")
+        extra["paged_decode"] = dict(workload=r2["name"], us_per_call=r2["ms_per_step"] * 1e3, gbs=r2["gbs"],
+                                     pct_of_hbm_peak=100 * r2["gbs"] / HBM_PEAK_GBS, kernel_us=r2["kernel_ms"] * 1e3,
+                                     bytes=r2["bytes"])
+        del r2
+        torch.cuda.empty_cache()
+        r4 = bench_appendkv(args, torch, fmha, gen, 100, 10)
+        extra["appendkv"] = dict(workload=r4["name"], us_per_call=r4["us_per_call"], bytes=r4["bytes"],
+                                 new_tokens=r4["new_tokens"])
+        for d in (128, 256):
+            r5 = bench_prefill(args, torch, fmha, gen, d, 10, 3)
+            extra[f"prefill_d{d}"] = dict(workload=r5["name"], ms_per_call=r5["ms_per_step"], tflops=r5["tflops"],
+                                          mfma_util_pct=100 * r5["tflops"] / MFMA_BF16_PEAK_TFLOPS, flops=r5["flops"],
+                                          kernel_ms=r5["kernel_ms"])
+
+    line = {
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic", "config": {"workload": name, "kv_pool_copies_rotated": args.copies},
+        "roofline": roof, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
