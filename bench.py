@@ -27,11 +27,14 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="splitkv", choices=["splitkv", "paged_decode", "prefill", "prefill256"],
+    ap.add_argument("--workload", default="splitkv", choices=["splitkv", "paged_decode", "prefill", "prefill256", "copy"],
                     help="workload of the headline line (default: split-KV long-context decode)")
     ap.add_argument("--copies", type=int, default=4, help="KV pool copies rotated between steps")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--kv-len", type=int, default=32768, help="KV length of the split-KV workload (study runs only)")
+    ap.add_argument("--no-shuffle", action="store_true", help="identity page order (study runs only)")
+    ap.add_argument("--num-splits", type=int, default=8, help="split count of the split-KV workload (study runs only)")
     return ap.parse_args()
 
 
@@ -56,9 +59,9 @@ def time_steps(fn, steps, warmup, torch, kernel_events=False):
 
 def bench_decode(args, torch, fmha, gen, which):
     if which == "splitkv":
-        w = gen.workload_splitkv_decode()
+        w = gen.workload_splitkv_decode(kv_len=args.kv_len, num_splits=args.num_splits, shuffle=not args.no_shuffle)
         ns = w["num_splits"]
-        name = "split-KV long-context decode: B=4 q=1 Hq64/Hk8 D128 L=32768 P=128 ns=8 + combine (bf16)"
+        name = f"split-KV long-context decode: B=4 q=1 Hq64/Hk8 D128 L={args.kv_len} P=128 ns={ns} + combine (bf16)"
     else:
         w = gen.workload_paged_decode()
         ns = fmha.num_splits_heuristic(32, 32, 8, 1, max(w["lens"]), 128)
@@ -169,6 +172,15 @@ def main():
     torch.cuda.set_device(0)
 
     extra = {}
+    if args.workload == "copy":
+        # calibration run for the hardware counters: a plain device copy of known size (512 MiB read + 512 MiB written)
+        n = 512 << 20
+        src = torch.full((n,), 1, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        wall, _ = time_steps(lambda i, ev: dst.copy_(src), args.steps, args.warmup, torch)
+        print(json.dumps({"metric": "device copy (counter calibration)", "value": 2 * n / (wall / args.steps) / 1e9,
+                          "unit": "GB/s", "bytes_read": n, "bytes_written": n, "steps": args.steps}))
+        return
     if args.workload in ("splitkv", "paged_decode"):
         r = bench_decode(args, torch, fmha, gen, args.workload)
         value, unit, metric = r["gbs"], "GB/s", "paged-KV decode HBM GB/s (% of peak) + us/call; prefill TFLOP/s, MFMA util %"

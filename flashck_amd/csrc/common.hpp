@@ -88,6 +88,50 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(const void FCK_LDS* p)
     return __builtin_bit_cast(u32x2_t, v);
 }
 
+// Cross-lane reductions on the VALU (v_permlane16_swap / v_permlane32_swap, no LDS round trip).
+// v_permlane32_swap a, b exchanges lanes 32..63 of a with lanes 0..31 of b; v_permlane16_swap does the same between the
+// odd 16-lane rows of a and the even rows of b.  Started from two copies of x they leave (x[l % 32], x[l % 32 + 32]) resp.
+// (x[even row of l], x[odd row of l]) in every lane.  The instructions are written as inline assembly because they
+// update both operands in place; the s_nop covers the wait states a VALU write needs before a lane permute reads it.
+__device__ __forceinline__ void swap32(float x, float& a, float& b)
+{
+    a = x;
+    b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap16(float x, float& a, float& b)
+{
+    a = x;
+    b = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+// over the lane pair (l, l ^ 32)
+__device__ __forceinline__ float pair32_max(float x)
+{
+    float a, b;
+    swap32(x, a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float pair32_sum(float x)
+{
+    float a, b;
+    swap32(x, a, b);
+    return a + b;
+}
+// over the four lanes that share l % 16
+__device__ __forceinline__ float quad16_max(float x)
+{
+    float a, b;
+    swap16(x, a, b);
+    return pair32_max(fmaxf(a, b));
+}
+__device__ __forceinline__ float quad16_sum(float x)
+{
+    float a, b;
+    swap16(x, a, b);
+    return pair32_sum(a + b);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -5,13 +5,17 @@
 //           16*MB packed query rows (query index, head-in-group) that share that KV head.
 //   waves = NW per workgroup; wave w walks the 32-key tiles w, w+NW, ... of the split with its own online-softmax
 //           state; the NW partial states are merged through LDS at the end.
-// Data path per 32-key tile and wave
-//   K   global -> VGPR directly in MFMA operand order (16 keys x 64 B per load instruction);
-//   V   global -> VGPR with whole 2*D-byte rows per 16*D/128 lanes, staged in a wave-private, XOR-swizzled LDS tile
-//       and read back transposed (ds_read_b64_tr_b16) as the A operand of O^T += V^T . P^T;
+// Data path per step (one 32-key tile per wave)
+//   K, V  global -> VGPR with whole 2*D-byte rows per D/8 lanes (every 128-byte line is touched by one instruction).
+//       Waves work in pairs: the even wave fetches the K rows of both tiles of the pair (64 consecutive keys), the odd
+//       wave fetches the V rows, so every wave streams from one array in bursts of 2*D/16 loads - measured to be the
+//       access shape the HBM system sustains best, whereas one wave alternating between the K and the V pool is
+//       15-20 % slower.  The rows are staged in per-wave, XOR-swizzled LDS tiles; K is read back with ds_read_b128
+//       as the A operand of S^T = K . Q^T, V is read back transposed (ds_read_b64_tr_b16) as the A operand of
+//       O^T += V^T . P^T;
 //   S^T = K . Q^T with v_mfma_f32_16x16x32, so that each lane keeps the scores of one query row and the
 //       probabilities it produces are already laid out as the B operand of the second product.
-// Loads of tile i+1 are issued before the arithmetic of tile i.
+// The loads of step i+1 are in flight while step i is computed from LDS.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -34,7 +38,7 @@ template <int D, int NW>
 constexpr size_t decode_lds_bytes()
 {
     typedef DecodeShape<D> S;
-    const size_t stage = (size_t)NW * S::VTILE;
+    const size_t stage = (size_t)NW * 2 * S::VTILE;
     const size_t merge = (size_t)NW * 16 * S::OSTRIDE * 4 + (size_t)NW * 2 * 16 * 4;
     return stage > merge ? stage : merge;
 }
@@ -147,65 +151,101 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
     const int last_key = sk_b - 1;
 
     // per-lane constants of the V staging tile
-    char FCK_LDS* vstage = (char FCK_LDS*)(smem) + wave * S::VTILE;
-    int vw_off[S::VN];
+    char FCK_LDS* kstage = (char FCK_LDS*)(smem) + wave * 2 * S::VTILE;
+    char FCK_LDS* vstage = kstage + S::VTILE;
+    int vw_off[S::VN], kw_off[S::VN];
 #pragma unroll
     for (int u = 0; u < S::VN; ++u) {
         const int key = u * S::KPI + lane / S::LPR;
         const int chunk = lane % S::LPR;
         vw_off[u] = key * S::VROW + ((chunk ^ v_swizzle<S::LPR>(key)) << 4);
+        kw_off[u] = key * S::VROW + ((chunk ^ (key & 7)) << 4);
     }
+    // K as the A operand: lane (key = nb * 16 + l16, k-group kg) reads chunk t * 4 + kg of its key row
+    const int kr_off = l16 * S::VROW;
+    const int kr_sw = l16 & 7;
     const int tr_key = kg * 4 + (l16 >> 2);
     const int tr_sw = v_swizzle<S::LPR>(tr_key);
     const int tr_base = tr_key * S::VROW + ((l16 & 2) << 3) + ((l16 & 1) << 3);
 
+    // ---- loading roles -------------------------------------------------------------------------------------------
+    // pair p = waves (2p, 2p+1); in step `it` they own tiles tA = t_begin + 2p + it * NW and tA + 1
+    const int role = wave & 1;         // 0: fetches K for the pair, 1: fetches V
+    const int pair0 = wave & ~1;       // even wave of the pair
+    const int n_iter = (t_end - t_begin + NW - 1) / NW;  // steps of the workgroup (uniform)
+    const uint16_t* src = role ? vp : kp;
+    char FCK_LDS* stageA = (char FCK_LDS*)(smem) + pair0 * 2 * S::VTILE + role * S::VTILE;  // tile of wave 2p
+    char FCK_LDS* stageB = stageA + 2 * S::VTILE;                                           // tile of wave 2p+1
+
     struct Frag {
-        u32x4_t k[2][S::KT];
-        u32x4_t v[S::VN];
+        u32x4_t a[2 * S::VN];
     };
 
-    auto load_tile = [&](int tile, Frag& f) {
-        const int kb = tile * S::TK;
-        if constexpr (kUniformPage) {
-            // the whole tile lies in one page (or the cache is contiguous): one row base per tile
-            const int kbc = min(kb, last_key);
-            const int64_t row0 = kv_row(a.kv, ks, kbc) - (kbc - kb);
-            const int room = last_key - kb;  // largest valid local key
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                const int kl = min(nb * 16 + l16, room);
-                const uint16_t* p = kp + (row0 + kl) * krow_stride + hkv * D + kg * 8;
-#pragma unroll
-                for (int t = 0; t < S::KT; ++t) f.k[nb][t] = ldg16(p + t * 32);
-            }
-#pragma unroll
-            for (int u = 0; u < S::VN; ++u) {
-                const int kl = min(u * S::KPI + lane / S::LPR, room);
-                f.v[u] = ldg16(vp + (row0 + kl) * krow_stride + hkv * D + (lane % S::LPR) * 8);
-            }
-        } else {
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                const int key = min(kb + nb * 16 + l16, last_key);
-                const uint16_t* p = kp + kv_row(a.kv, ks, key) * krow_stride + hkv * D + kg * 8;
-#pragma unroll
-                for (int t = 0; t < S::KT; ++t) f.k[nb][t] = ldg16(p + t * 32);
-            }
-#pragma unroll
-            for (int u = 0; u < S::VN; ++u) {
-                const int key = min(kb + u * S::KPI + lane / S::LPR, last_key);
-                f.v[u] = ldg16(vp + kv_row(a.kv, ks, key) * krow_stride + hkv * D + (lane % S::LPR) * 8);
-            }
+    // Page ids of the pair's tiles, 64 steps at a time: lane j holds the pages of step it0 + j, so the loop reads them
+    // with v_readlane instead of a dependent scalar load per step.
+    int page_regA = 0, page_regB = 0;
+    auto page_index = [&](int key) { return a.kv.page_shift >= 0 ? key >> a.kv.page_shift : key / a.kv.page_size; };
+    auto clamp_tile = [&](int t) { return min(t, t_end - 1); };
+    auto fetch_pages = [&](int it0) {
+        const int it = it0 + lane;
+        if (ks.table != nullptr && it < n_iter) {
+            const int tA = t_begin + pair0 + it * NW;
+            page_regA = ks.table[page_index(clamp_tile(tA) * S::TK)];
+            page_regB = ks.table[page_index(clamp_tile(tA + 1) * S::TK)];
         }
     };
 
-    auto compute_tile = [&](int tile, const Frag& f) {
-        const int kb = tile * S::TK;
-        // stage V (wave private): write rows, then read them back transposed
+    auto load_step = [&](int it, Frag& f) {
+        if constexpr (kUniformPage) {
+            if ((it & 63) == 0) fetch_pages(it);
+        }
 #pragma unroll
-        for (int u = 0; u < S::VN; ++u) *(u32x4_t FCK_LDS*)(vstage + vw_off[u]) = f.v[u];
+        for (int half = 0; half < 2; ++half) {
+            const int tile = clamp_tile(t_begin + pair0 + half + it * NW);
+            const int kb = tile * S::TK;
+            if constexpr (kUniformPage) {
+                // the whole tile lies in one page (or the cache is contiguous): one row base per tile
+                int64_t row0;
+                if (ks.table != nullptr) {
+                    const int page = __builtin_amdgcn_readlane(half ? page_regB : page_regA, it & 63);
+                    row0 = (int64_t)page * a.kv.page_size + (kb - page_index(kb) * a.kv.page_size);
+                } else {
+                    row0 = ks.base_row + kb;
+                }
+                const int room = last_key - kb;  // largest valid local key
+#pragma unroll
+                for (int u = 0; u < S::VN; ++u) {
+                    const int kl = min(u * S::KPI + lane / S::LPR, room);
+                    f.a[half * S::VN + u] = ldg16(src + (row0 + kl) * krow_stride + hkv * D + (lane % S::LPR) * 8);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < S::VN; ++u) {
+                    const int key = min(kb + u * S::KPI + lane / S::LPR, last_key);
+                    f.a[half * S::VN + u] = ldg16(src + kv_row(a.kv, ks, key) * krow_stride + hkv * D + (lane % S::LPR) * 8);
+                }
+            }
+        }
+    };
+    auto store_step = [&](const Frag& f) {
+#pragma unroll
+        for (int u = 0; u < S::VN; ++u) {
+            const int off = role ? vw_off[u] : kw_off[u];
+            *(u32x4_t FCK_LDS*)(stageA + off) = f.a[u];
+            *(u32x4_t FCK_LDS*)(stageB + off) = f.a[S::VN + u];
+        }
+    };
+
+    auto compute_tile = [&](int it) {
+        const int kb = (t_begin + wave + it * NW) * S::TK;
 
         // S^T[key][row] = K . Q^T
+        u32x4_t kfrag[2][S::KT];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int t = 0; t < S::KT; ++t)
+                kfrag[nb][t] = *(const u32x4_t FCK_LDS*)(kstage + nb * 16 * S::VROW + kr_off + (((t * 4 + kg) ^ kr_sw) << 4));
         f32x4_t s[MB][2];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
@@ -213,7 +253,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
             for (int nb = 0; nb < 2; ++nb) {
                 f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int t = 0; t < S::KT; ++t) acc = T::mfma16(as_vec8<vec8>(f.k[nb][t]), qf[mb][t], acc);
+                for (int t = 0; t < S::KT; ++t) acc = T::mfma16(as_vec8<vec8>(kfrag[nb][t]), qf[mb][t], acc);
                 s[mb][nb] = acc;
             }
 
@@ -232,8 +272,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
                     x[nb * 4 + j] = v;
                     tmax = fmaxf(tmax, v);
                 }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            tmax = quad16_max(tmax);
             const float m_new = fmaxf(m_run[mb], tmax);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
             const float alpha = fast_exp2(m_run[mb] - m_use);
@@ -257,8 +296,6 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
         }
 
         // O^T[dv][row] += V^T . P^T
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int db = 0; db < S::DB; ++db) {
             const int coff = tr_base + ((((db * 2) ^ tr_sw)) << 4);
@@ -268,34 +305,35 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) oacc[mb][db] = T::mfma16(as_vec8<vec8>(av), pf[mb], oacc[mb][db]);
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
     };
 
-    {
-        int tile = t_begin + wave;
-        if (tile < t_end) {
-            Frag cur;
-            load_tile(tile, cur);
-            while (true) {
-                const int nxt = tile + NW;
-                const bool more = nxt < t_end;
-                Frag pre;
-                if (more) load_tile(nxt, pre);
-                compute_tile(tile, cur);
-                if (!more) break;
-                cur = pre;
-                tile = nxt;
-            }
+    // Software pipeline over the steps of the workgroup.  The last step is peeled so that the prefetch is unconditional
+    // inside the loop (a conditional prefetch makes the wait counters at the join cover both paths, which serialises
+    // load and compute).  Two workgroup barriers per step: all tiles read / next tiles written.
+    if (n_iter > 0) {
+        {
+            Frag f0;
+            load_step(0, f0);
+            store_step(f0);
         }
+        __syncthreads();
+        int it = 0;
+        for (; it + 1 < n_iter; ++it) {
+            Frag pre;
+            load_step(it + 1, pre);
+            if (t_begin + wave + it * NW < t_end) compute_tile(it);
+            __syncthreads();
+            store_step(pre);
+            __syncthreads();
+        }
+        if (t_begin + wave + it * NW < t_end) compute_tile(it);
     }
 
     // ---- merge the NW partial states --------------------------------------------------------------------------
     // each lane owns a partial row sum over its 8 key slots per tile: fold the 4 lanes of a row
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-        l_run[mb] += __shfl_xor(l_run[mb], 16);
-        l_run[mb] += __shfl_xor(l_run[mb], 32);
+        l_run[mb] = quad16_sum(l_run[mb]);
     }
 
     float* obuf = reinterpret_cast<float*>(smem);                       // [NW][16][OSTRIDE]

@@ -32,7 +32,8 @@ def rotary_tables(max_pos: int, rotary_dim: int, dtype, base: float = 10000.0):
     return torch.cos(ang).to(dtype).contiguous(), torch.sin(ang).to(dtype).contiguous()
 
 
-def paged_layout(lens: Sequence[int], page_size: int, g, slack: float = 0.10, capacity: Optional[Sequence[int]] = None):
+def paged_layout(lens: Sequence[int], page_size: int, g, slack: float = 0.10, capacity: Optional[Sequence[int]] = None,
+                 shuffle: bool = True):
     """Shuffled block table: sequence b takes consecutive entries of a random permutation of the pool.
 
     Returns (block_table int32 [B, max_pages], num_pool_pages).  `capacity` (>= lens) reserves pages for growth.
@@ -42,6 +43,8 @@ def paged_layout(lens: Sequence[int], page_size: int, g, slack: float = 0.10, ca
     total = sum(pages)
     pool = int(math.ceil(total * (1.0 + slack)))
     perm = torch.randperm(pool, generator=g).to(torch.int32)
+    if not shuffle:
+        perm = torch.arange(pool, dtype=torch.int32)
     table = torch.zeros(len(lens), max(pages), dtype=torch.int32)
     at = 0
     for b, n in enumerate(pages):
@@ -65,9 +68,9 @@ def scatter_to_pages(rows: List[torch.Tensor], table: torch.Tensor, pool: int, p
     return cache
 
 
-def paged_kv(lens, hk, d, dtype, g, page_size=128, slack=0.10, capacity=None):
+def paged_kv(lens, hk, d, dtype, g, page_size=128, slack=0.10, capacity=None, shuffle=True):
     """Random K/V for sequences of the given lengths, stored in a shuffled paged cache with NaN in unused slots."""
-    table, pool = paged_layout(lens, page_size, g, slack, capacity)
+    table, pool = paged_layout(lens, page_size, g, slack, capacity, shuffle)
     k_rows = [randn((n, hk, d), dtype, g) for n in lens]
     v_rows = [randn((n, hk, d), dtype, g) for n in lens]
     k_cache = scatter_to_pages(k_rows, table, pool, page_size)
@@ -106,11 +109,11 @@ def workload_paged_decode(seed=BASE_SEED + 2, batch=32, hq=32, hk=8, head_dim=12
 
 
 def workload_splitkv_decode(seed=BASE_SEED + 3, batch=4, hq=64, hk=8, head_dim=128, kv_len=32768, page_size=128,
-                            num_splits=8, dtype=torch.bfloat16):
+                            num_splits=8, dtype=torch.bfloat16, shuffle=True):
     """3: split-KV long-context decode, fixed KV length, shuffled pages, num_splits partials + combine."""
     g = _gen(seed)
     lens = [kv_len] * batch
-    kv = paged_kv(lens, hk, head_dim, dtype, g, page_size)
+    kv = paged_kv(lens, hk, head_dim, dtype, g, page_size, shuffle=shuffle)
     kv["q"] = randn((batch, 1, hq, head_dim), dtype, g)
     kv["scale"] = 1.0 / math.sqrt(head_dim)
     kv["num_splits"] = num_splits

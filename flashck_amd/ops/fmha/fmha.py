@@ -185,11 +185,11 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
 
 def fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype, cu_seqlens_q=None, max_seqlen_q: int = 0, out=None) -> torch.Tensor:
     """LSE combine of split-KV partials -> o [B,sq,Hq,Dv] (or [total_q,Hq,Dv] in group mode)."""
+    if dtype not in _DTYPE_ID:
+        raise TypeError(f"FMHA supports torch.float16 and torch.bfloat16, got {dtype}")
     _check_tensor("lse_acc", lse_acc, dtype=torch.float32, ndim=4)
     _check_tensor("o_acc", o_acc, dtype=torch.float32, ndim=5)
     _check_tensor("cu_seqlens_q", cu_seqlens_q, dtype=torch.int32, optional=True)
-    if dtype not in _DTYPE_ID:
-        raise TypeError(f"FMHA supports torch.float16 and torch.bfloat16, got {dtype}")
     bs, Hq, ns, sq, Dv = o_acc.shape
     if tuple(lse_acc.shape) != (bs, Hq, ns, sq):
         raise ValueError(f"lse_acc {tuple(lse_acc.shape)} does not match o_acc {tuple(o_acc.shape)}")

@@ -1,0 +1,107 @@
+"""CPU-only checks of the boundary: the built library exports every symbol the header declares, argument validation
+answers with error codes and messages before any launch, and the Python operators validate like the reference's."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from flashck_amd import _lib
+from flashck_amd.ops import fmha
+from flashck_amd.utils import FlashCKOperationType, get_flashck_functions, is_available
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "flashck", "fmha", "fmha_c_api.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return re.findall(r"FCK_EXPORT\s+[\w\s\*]+?\b(fck_\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 10
+    assert set(names) == set(_lib.SIGNATURES), "ctypes signature table and header disagree"
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_registry_has_fmha():
+    assert is_available(FlashCKOperationType.FMHA.value)
+    fns = get_flashck_functions("fmha")
+    for k in ("forward", "forward_splitkv", "forward_splitkv_combine", "forward_appendkv", "batch_prefill", "forward_pagedkv"):
+        assert callable(fns[k])
+    assert not is_available(FlashCKOperationType.LAYER_NORM.value)
+
+
+def test_error_codes_without_a_gpu():
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    # unsupported dtype
+    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, 7, None)
+    assert rc == -2 and b"dtype" in lib.fck_last_error()
+    # Hq not a multiple of Hk
+    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 3, 2, 64, 64, 8, 0.125, -1, -1, 0, 4, None)
+    assert rc == -1 and b"multiple" in lib.fck_last_error()
+    # unsupported head dim
+    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 80, 80, 8, 0.125, -1, -1, 0, 4, None)
+    assert rc == -2 and b"head_dim" in lib.fck_last_error()
+    # null pointer
+    rc = lib.fck_fmha_fwd(None, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, 4, None)
+    assert rc == -1 and b"null" in lib.fck_last_error()
+    # bias is declared by the signature but has no kernel
+    rc = lib.fck_fmha_fwd(p, p, p, p, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, 4, None)
+    assert rc == -2 and b"bias" in lib.fck_last_error()
+    # misaligned pointer
+    q = ctypes.c_void_p(p.value + 2)
+    rc = lib.fck_fmha_fwd(q, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, 4, None)
+    assert rc == -1 and b"aligned" in lib.fck_last_error()
+    # split-KV: bad split count, paged cache without key counts
+    rc = lib.fck_fmha_fwd_splitkv(p, p, p, None, p, p, None, None, None, None, None, 1, 1, 8, 2, 2, 64, 64, 1, 0, 0, 0,
+                                  0.125, -1, -1, 0, 4, None)
+    assert rc == -1 and b"num_splits" in lib.fck_last_error()
+    rc = lib.fck_fmha_fwd_splitkv(p, p, p, None, p, p, None, None, None, p, None, 1, 1, 8, 2, 2, 64, 64, 1, 2, 4, 16,
+                                  0.125, -1, -1, 0, 4, None)
+    assert rc == -1 and b"key counts" in lib.fck_last_error()
+    # combine: bad head dim; appendkv: odd rotary_dim
+    rc = lib.fck_fmha_fwd_splitkv_combine(p, p, p, None, 1, 1, 2, 96, 1, 2, 4, None)
+    assert rc == -2
+    rc = lib.fck_fmha_fwd_appendkv(None, p, p, p, p, p, None, 1, p, p, 31, 2, 1, p, 4, 16, None, 0, 1, 2, 2, 64, 64, 4, None)
+    assert rc == -1 and b"rotary_dim" in lib.fck_last_error()
+    # mask type out of range
+    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 9, 4, None)
+    assert rc == -1 and b"mask_type" in lib.fck_last_error()
+
+
+def test_workspace_bytes_and_heuristic():
+    lib = _lib.load()
+    # o_acc [B,Hq,ns,sq,Dv] fp32 + lse_acc [B,Hq,ns,sq] fp32
+    assert lib.fck_fmha_splitkv_workspace_bytes(4, 64, 1, 128, 8) == 4 * 64 * 8 * 1 * 128 * 4 + 4 * 64 * 8 * 4
+    assert lib.fck_fmha_splitkv_workspace_bytes(0, 64, 1, 128, 8) == 0
+    # long context, few sequences: split; many workgroups already or short context: do not
+    assert fmha.num_splits_heuristic(4, 64, 8, 1, 32768, 128, 256) >= 8
+    assert fmha.num_splits_heuristic(256, 32, 8, 1, 4096, 128, 256) == 1
+    assert fmha.num_splits_heuristic(1, 8, 8, 1, 200, 128, 256) == 1
+    for args in [(1, 8, 1, 1, 10 ** 6, 128, 256), (32, 32, 8, 1, 4096, 128, 256)]:
+        assert 1 <= fmha.num_splits_heuristic(*args) <= 128
+
+
+def test_python_validation_mirrors_reference_errors():
+    q = torch.zeros(1, 4, 2, 64, dtype=torch.float16)
+    with pytest.raises(TypeError):
+        fmha.fmha_fwd("q", q, q)
+    with pytest.raises(ValueError):   # CPU tensors never reach the GPU path and there is no fallback
+        fmha.fmha_fwd(q, q, q)
+    with pytest.raises(TypeError):
+        fmha.fmha_fwd_splitkv_combine(torch.zeros(1, 2, 1, 4), torch.zeros(1, 2, 1, 4, 64), torch.float32)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libflashck_fmha.so"))
+    with pytest.raises(_lib.FlashCKLibraryError):
+        _lib.load()
