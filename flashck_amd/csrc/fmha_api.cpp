@@ -255,9 +255,17 @@ int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* kne
 }
 
 static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t q_max_seq_len, bool uniform, void* stream,
-                          const char* what)
+                          const char* what, int64_t max_keys_per_seq)
 {
+    // the ping-pong kernel keeps one page id per key tile in LDS
+    const bool pp_uniform = uniform && max_keys_per_seq <= (int64_t)fck::kPrefillPageCache * fck::kPrefillKeyTile;
     if (q_max_seq_len <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_max_seq_len must be positive");
+    // Long query runs at head dim <= 128 take the 8-wave ping-pong kernel (256 rows per workgroup); short runs and
+    // head dim 256 take the 4-wave kernel (128 rows per workgroup).
+    if (d <= 128 && q_max_seq_len > 128) {
+        a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
+        return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, pp_uniform, static_cast<hipStream_t>(stream)), what);
+    }
     a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
     return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
 }
@@ -299,7 +307,7 @@ int fck_fmha_fwd(const void* q, const void* k, const void* v, const void* bias, 
         a.kv.seqlen_k_ptr = seqlen_k_ptr;
         if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
     }
-    return prefill_common(a, d, dtype, q_max_seq_len, true, stream, "FmhaFwd launch");
+    return prefill_common(a, d, dtype, q_max_seq_len, true, stream, "FmhaFwd launch", 0);
 }
 
 int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
@@ -335,7 +343,8 @@ int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cac
     a.kv.kv_last_page_lens = kv_last_page_lens;
     a.kv.page_size = (int32_t)page_block_size;
     a.kv.page_shift = log2_exact(page_block_size);
-    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdBatchPrefill launch");
+    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdBatchPrefill launch",
+                          num_total_pages * page_block_size);
 }
 
 int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
@@ -374,7 +383,8 @@ int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache
     a.kv.page_size = (int32_t)page_block_size;
     a.kv.page_shift = log2_exact(page_block_size);
     if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
-    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdPagedKV launch");
+    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdPagedKV launch",
+                          batch_stride_block_table * page_block_size);
 }
 
 }  // extern "C"

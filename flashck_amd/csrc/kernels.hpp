@@ -67,5 +67,11 @@ hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int row
 hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st);
 hipError_t launch_appendkv(const AppendKvArgs& a, int dtype, int max_new, hipStream_t st);
 hipError_t launch_prefill(const PrefillArgs& a, int d, int dtype, bool uniform_page, hipStream_t st);
+// Tiles of a sequence whose page ids the ping-pong prefill kernel caches in LDS; with more tiles than this the caller
+// must pass uniform_page = false (per-row table lookups).
+constexpr int kPrefillPageCache = 4096;
+constexpr int kPrefillKeyTile = 64;
+// 256-row workgroups (a.m_tiles counts 256-row tiles); head dims 64 and 128
+hipError_t launch_prefill_pingpong(const PrefillArgs& a, int d, int dtype, bool uniform_page, hipStream_t st);
 
 }  // namespace fck

@@ -211,24 +211,32 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
         for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
             for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        tmax = pair32_max(tmax);
         tmax *= a.scale_log2;  // scale > 0: max commutes with the scaling
-        const float m_new = fmaxf(m_run, tmax);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run - m_use);
-        m_run = m_new;
+        // Lazy rescale: the running reference m_run only moves when some row's maximum outgrows it by more than
+        // kLazy (in log2 units).  Softmax is shift invariant, so keeping a stale reference is exact; it bounds the
+        // exponentials by 2^kLazy and saves the accumulator rescale on almost every tile.
+        constexpr float kLazy = 8.f;
+        if (__builtin_amdgcn_ballot_w64(tmax > m_run + kLazy) != 0) {
+            const float m_new = fmaxf(m_run, tmax);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = fast_exp2(m_run - m_use);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int i = 0; i < S::DVB; ++i) oacc[i] *= alpha;
+        }
+        const float m_ref = (m_run == -INFINITY) ? 0.f : m_run;
         float psum = 0.f;
 #pragma unroll
         for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
-                const float p = fast_exp2(__builtin_fmaf(s[mbk][j], a.scale_log2, -m_use));
+                const float p = fast_exp2(__builtin_fmaf(s[mbk][j], a.scale_log2, -m_ref));
                 s[mbk][j] = p;
                 psum += p;
             }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int i = 0; i < S::DVB; ++i) oacc[i] *= alpha;
+        l_run += psum;
 
         // ---- O^T += V^T . P^T ---------------------------------------------------------------------------------------
 #pragma unroll
@@ -256,7 +264,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
     }
 
     // ---- epilogue ----------------------------------------------------------------------------------------------------
-    l_run += __shfl_xor(l_run, 32);
+    l_run = pair32_sum(l_run);
     if (row_ok) {
         const float inv = (l_run == 0.f) ? 0.f : 1.f / l_run;
         uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * D;
