@@ -6,18 +6,25 @@
 //   grid  = 1-D, XCD-aware order; a workgroup of 8 waves owns 256 query rows of one head: group g = wave / 4 owns rows
 //           [g*128, g*128+128), 32 rows per wave.  Waves w and w+4 sit on the same SIMD.
 // Phases (one workgroup barrier after each); tile i = the i-th key tile of the visible range
-//   group 0, phase 2i   : matrix phase  M(i) = { O^T += V^T.P^T of tile i-1 ; S^T = K.Q^T of tile i }
-//   group 0, phase 2i+1 : vector phase  V(i) = { online softmax of tile i: S -> P }
-//   group 1 runs the same instruction stream one phase later (it passes one extra barrier before its first matrix
-//   phase, group 0 one extra after its last), so every phase pairs one M with one V on each SIMD and no branch inside
-//   the loop depends on the group.
+//   matrix phase  M(i) = { O^T += V^T.P^T of tile i ; S^T = K.Q^T of tile i+1 }
+//   vector phase  V(i) = { online softmax of tile i: S -> P }
+//   group 0 runs M(i) in phase 2i+2 and V(i) in phase 2i+1; group 1 runs the same instruction stream one phase later
+//   (it passes one extra barrier before its first matrix phase, group 0 one extra after its last), so every phase pairs
+//   one M with one V on each SIMD and no branch inside the loop depends on the group.
 // Data path
-//   K, V tiles: global -> VGPR (whole rows, 16 B per lane) -> swizzled LDS, two buffers each; the loads of a tile are
-//   issued six phases (three tiles) before they are written to LDS.  K is read with ds_read_b128 as the A operand of
-//   v_mfma_f32_32x32x16, V with the transposing ds_read_b64_tr_b16; Q is parked in LDS; P never leaves registers
-//   because the accumulator layout of the first product is the B-operand layout of the second.
+//   K, V tiles: global -> LDS directly (global_load_lds_dwordx4, 1 KiB per wave instruction), rings of kRing buffers
+//   each; the XOR swizzle of the staged tile is applied on the global side (lane l of an instruction always lands at
+//   LDS byte l*16 of its block, so it fetches the chunk that belongs there).  In M(i) every wave requests its share of
+//   K_{i+3} and V_{i+2} into the buffers M(i-1) was the last to read, and before the barrier that ends M(i) it waits
+//   until its share of K_{i+2} and V_{i+1} has landed.  No register is a load destination, so nothing the compiler
+//   schedules can wait on these loads by accident.  K is read with ds_read_b128 as the A operand of
+//   v_mfma_f32_32x32x16, V with the transposing ds_read_b64_tr_b16, both two MFMA pairs ahead of their use; Q stays in
+//   registers; P never leaves registers because the accumulator layout of the first product is the B-operand layout of
+//   the second.
 #include "common.hpp"
 #include "kernels.hpp"
+
+#include <type_traits>
 
 namespace fck {
 
@@ -31,8 +38,9 @@ struct PPShape {
     static constexpr int ROWB = D * 2;  // bytes per staged row
     static constexpr int CH = D / 8;    // 16-byte chunks per row
     static constexpr int TILEB = BN * ROWB;
-    static constexpr int NCH = BN * CH;                    // 16-byte chunks per tile
-    static constexpr int LD = (NCH + 511) / 512;           // 16-byte loads per thread and tile (threads past NCH idle)
+    static constexpr int LD = TILEB / 1024 / 8;  // 1 KiB global->LDS instructions per wave and tile
+    static constexpr int RING = 3;               // LDS buffers per operand
+    static_assert(TILEB % 8192 == 0, "a tile is split evenly over the 8 waves");
 };
 
 // XOR swizzles of the 16-byte chunk index.  They keep both LDS read patterns free of bank conflicts whether the LDS
@@ -60,8 +68,12 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
 {
     typedef PPShape<D, BN> S;
     typedef typename T::vec8 vec8;
+    static_assert(S::NB == 2, "the matrix phase is written for 64-key tiles");
+    constexpr int kRing = S::RING;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    char FCK_LDS* lds = (char FCK_LDS*)smem;  // K0 | K1 | V0 | V1 | Q fragments (8 waves x KT x 1 KiB) | page ids (kPrefillPageCache x int32)
+    char FCK_LDS* lds = (char FCK_LDS*)smem;  // K ring | V ring | page ids (kPrefillPageCache x int32)
+    char FCK_LDS* const k_ring = lds;
+    char FCK_LDS* const v_ring = lds + kRing * S::TILEB;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -121,17 +133,14 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     const int n = t_end - t_begin;  // number of tiles (may be <= 0)
 
     // ---- Q fragments (B operand of S^T = K . Q^T): lane (row = l32, k-group = half) ------------------------------
-    // They are parked in a wave-private LDS area, lane-linear, and re-read in every matrix phase: the 4*KT registers
-    // they would occupy are what lets three K/V tiles be in flight from global memory.
-    char FCK_LDS* qlds = lds + 4 * S::TILEB + wave * (S::KT * 1024) + lane * 16;
+    u32x4_t qf[S::KT];
     {
         const uint16_t* qp =
             reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * D + half * 8;
 #pragma unroll
         for (int t = 0; t < S::KT; ++t) {
-            u32x4_t v = {0u, 0u, 0u, 0u};
-            if (row_ok) v = ldg16(qp + t * 16);
-            *(u32x4_t FCK_LDS*)(qlds + t * 1024) = v;
+            qf[t] = u32x4_t{0u, 0u, 0u, 0u};
+            if (row_ok) qf[t] = ldg16(qp + t * 16);
         }
     }
 
@@ -149,27 +158,26 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     const int64_t row_stride = (int64_t)a.hk * D;
     const int last_key = sk_b - 1;
 
-    // global -> LDS copy assignment: 16-byte chunk (row, c) per thread and step
-    int cp_row[S::LD], cp_c[S::LD], cp_koff[S::LD], cp_voff[S::LD];
+    // global -> LDS assignment: wave w fills the 1 KiB blocks w, w+8, ... of a tile; lane l of an instruction lands at
+    // byte l*16 of its block, i.e. at (row, physical chunk) below, and fetches the logical chunk that the swizzle maps
+    // there.
+    int cp_row[S::LD], cp_k[S::LD], cp_v[S::LD];  // tile row, element offsets (row-relative) of the K and V chunk
 #pragma unroll
     for (int u = 0; u < S::LD; ++u) {
-        const int cid = min(tid + 512 * u, S::NCH - 1);  // threads past the tile repeat its last chunk (same bytes)
-        cp_row[u] = cid / S::CH;
-        cp_c[u] = cid % S::CH;
-        cp_koff[u] = cp_row[u] * S::ROWB + ((cp_c[u] ^ k_swz<D>(cp_row[u])) << 4);
-        cp_voff[u] = cp_row[u] * S::ROWB + ((cp_c[u] ^ v_swz<D>(cp_row[u], cp_c[u])) << 4);
+        const int off = (wave + 8 * u) * 1024 + lane * 16;
+        const int row = off / S::ROWB;
+        const int pc = (off % S::ROWB) >> 4;
+        cp_row[u] = row;
+        cp_k[u] = (pc ^ k_swz<D>(row)) * 8;
+        const int t = pc ^ ((row & 3) << 1);
+        cp_v[u] = (D >= 128 ? (t ^ (((t >> 1) & 1) << 3)) : t) * 8;  // inverse of lc -> lc ^ v_swz(row, lc)
     }
 
-    struct Regs {
-        u32x4_t k[S::LD], v[S::LD];
-    };
-
-    // Page ids (uniform-page path): the pages of this workgroup's tiles are copied into LDS once, so that the lookups
-    // of the main loop are LDS reads (lgkmcnt) and never wait on the vector loads in flight (vmcnt is shared by all
-    // global loads of a wave and counts in order).  The host only selects this path when a sequence cannot have more
-    // than kPrefillPageCache tiles.
+    // Page ids (uniform-page path): the pages of this workgroup's tiles are copied into LDS once, so the lookups of
+    // the main loop are LDS reads.  The host only selects this path when a sequence cannot have more than
+    // kPrefillPageCache tiles.
     constexpr int kPageCache = kPrefillPageCache;
-    int FCK_LDS* page_lds = (int FCK_LDS*)(lds + 4 * S::TILEB + 8 * S::KT * 1024);
+    int FCK_LDS* page_lds = (int FCK_LDS*)(lds + 2 * kRing * S::TILEB);
     auto page_index = [&](int key) __attribute__((always_inline)) {
         return a.kv.page_shift >= 0 ? key >> a.kv.page_shift : key / a.kv.page_size;
     };
@@ -185,31 +193,41 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         }
         return ks.base_row + kb;
     };
-    // Every step of the main loop requests exactly one K tile and one V tile, unconditionally (tile indices past the
-    // end are clamped and re-read the last tile): with a fixed number of loads per step the compiler can count how many
-    // younger loads may stay outstanding when a tile is written to LDS, instead of draining the counter to zero.
-    auto load_tile = [&](const uint16_t* base, int i, int64_t row0, u32x4_t (&dst)[S::LD]) __attribute__((always_inline)) {
+    auto tile = [&](int i) __attribute__((always_inline)) { return min(i, n - 1); };  // requests past the end re-read the last tile
+    // request this wave's share of local tile i into ring buffer `slot` (wave-uniform)
+    auto request = [&](const uint16_t* base, char FCK_LDS* ring, int slot_, int i, const int (&cp_c)[S::LD]) __attribute__((always_inline)) {
         const int kb = (t_begin + i) * S::BN;
-        if constexpr (kUniformPage) {
-            const int room = last_key - kb;
+        const int room = last_key - kb;
+        int64_t row0 = 0;
+        if constexpr (kUniformPage) row0 = tile_row0(i);
 #pragma unroll
-            for (int u = 0; u < S::LD; ++u)
-                dst[u] = ldg16(base + (row0 + min(cp_row[u], room)) * row_stride + hkv * D + cp_c[u] * 8);
-        } else {
-#pragma unroll
-            for (int u = 0; u < S::LD; ++u)
-                dst[u] = ldg16(base + kv_row(a.kv, ks, min(kb + cp_row[u], last_key)) * row_stride + hkv * D + cp_c[u] * 8);
+        for (int u = 0; u < S::LD; ++u) {
+            const int row = min(cp_row[u], room);  // rows past the last key repeat it (their scores are masked)
+            // Written as assembly on purpose: a load the compiler knows about makes it drain the whole load queue
+            // before the next LDS read it cannot prove disjoint.  m0 carries the LDS address of the block and is
+            // put back afterwards, since the compiler does not expect it to change.
+            uint32_t m0_saved;
+            const uint32_t dst = (uint32_t)(uintptr_t)(ring + slot_ * S::TILEB + (wave + 8 * u) * 1024);
+            if constexpr (kUniformPage) {
+                const uint16_t* tb = base + (row0 * row_stride + hkv * D);
+                const uint32_t off = (uint32_t)(row * (int)row_stride + cp_c[u]) * 2u;
+                asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
+                             : "=&s"(m0_saved)
+                             : "s"(dst), "v"(off), "s"(tb)
+                             : "memory");
+            } else {
+                const uint16_t* src = base + kv_row(a.kv, ks, kb + row) * row_stride + hkv * D + cp_c[u];
+                asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+                             : "=&s"(m0_saved)
+                             : "s"(dst), "v"(src)
+                             : "memory");
+            }
         }
     };
-    auto store_k = [&](int i, const Regs& R) __attribute__((always_inline)) {
-        char FCK_LDS* kd = lds + (i & 1) * S::TILEB;
-#pragma unroll
-        for (int u = 0; u < S::LD; ++u) *(u32x4_t FCK_LDS*)(kd + cp_koff[u]) = R.k[u];
-    };
-    auto store_v = [&](int i, const Regs& R) __attribute__((always_inline)) {
-        char FCK_LDS* vd = lds + (2 + (i & 1)) * S::TILEB;
-#pragma unroll
-        for (int u = 0; u < S::LD; ++u) *(u32x4_t FCK_LDS*)(vd + cp_voff[u]) = R.v[u];
+    // wait until at most `keep` of this wave's vector-memory operations are outstanding (they complete in order)
+    auto wait_vm = [&](auto keep) __attribute__((always_inline)) {
+        constexpr int N = decltype(keep)::value;
+        __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
     };
 
     // per-lane LDS read offsets
@@ -224,42 +242,65 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     const int v_rd = v_row * S::ROWB + ((i16 & 1) << 3);
     const int v_c0 = (q4 & 1) * 2 + ((i16 & 3) >> 1);  // chunk inside the 32-column block (4 chunks)
 
-    // S^T = K . Q^T of local tile i
-    auto qk = [&](int i) __attribute__((always_inline)) {
-        const char FCK_LDS* kt = lds + (i & 1) * S::TILEB;
+    // Matrix phase: O^T += V^T . P^T from the V tile in `vt` (when PV), then S^T = K . Q^T from the K tile in `kt`
+    // (when QK), as one sequence of steps of two MFMAs; the LDS operands of a step are requested two steps ahead.
+    constexpr int kPvSteps = 2 * S::NB * (S::DVB / 2);
+    auto matrix = [&](auto PV, auto QK, const char FCK_LDS* vt, const char FCK_LDS* kt) __attribute__((always_inline)) {
+        constexpr bool kPv = decltype(PV)::value, kQk = decltype(QK)::value;
+        constexpr int kP = kPv ? kPvSteps : 0;
+        constexpr int kSteps = kP + (kQk ? S::KT : 0);
+        u32x4_t bf[3][2];
+        auto fetch = [&](int m, u32x4_t (&d)[2]) __attribute__((always_inline)) {
+            if (m < kP) {
+                const int ks4 = m / (S::DVB / 2), pr = m % (S::DVB / 2);  // 16 keys ks4*16..+15; rows +{0,8}+v_row share v_row's swizzle
+                const char FCK_LDS* vb = vt + ks4 * 16 * S::ROWB + v_rd;
 #pragma unroll
-        for (int mbk = 0; mbk < S::NB; ++mbk)
+                for (int e = 0; e < 2; ++e) {
+                    const int lc = (pr * 2 + e) * 4 + v_c0;
+                    const int coff = ((lc ^ v_swz<D>(v_row, lc)) << 4);
+                    const u32x2_t lo4 = lds_read_tr16(vb + coff);
+                    const u32x2_t hi4 = lds_read_tr16(vb + 8 * S::ROWB + coff);
+                    d[e] = u32x4_t{lo4[0], lo4[1], hi4[0], hi4[1]};
+                }
+            } else {
+                const int t = m - kP;
 #pragma unroll
-            for (int j = 0; j < 16; ++j) s[mbk][j] = 0.f;
-#pragma unroll
-        for (int t = 0; t < S::KT; ++t) {
-            const vec8 qv = as_vec8<vec8>(*(const u32x4_t FCK_LDS*)(qlds + t * 1024));
-#pragma unroll
-            for (int mbk = 0; mbk < S::NB; ++mbk) {
-                const u32x4_t kv = *(const u32x4_t FCK_LDS*)(kt + mbk * 32 * S::ROWB + k_rd + (((t * 2 + half) ^ k_sw) << 4));
-                s[mbk] = T::mfma32(as_vec8<vec8>(kv), qv, s[mbk]);
+                for (int mbk = 0; mbk < 2; ++mbk)
+                    d[mbk] = *(const u32x4_t FCK_LDS*)(kt + mbk * 32 * S::ROWB + k_rd + (((t * 2 + half) ^ k_sw) << 4));
             }
-        }
-    };
-    // O^T += V^T . P^T of local tile i
-    auto pv = [&](int i) __attribute__((always_inline)) {
-        const char FCK_LDS* vt = lds + (2 + (i & 1)) * S::TILEB;
+        };
+        auto mma = [&](int m, const u32x4_t (&d)[2]) __attribute__((always_inline)) {
+            if (m < kP) {
+                const int ks4 = m / (S::DVB / 2), pr = m % (S::DVB / 2);
+                const vec8 pf = as_vec8<vec8>(pfrag[ks4]);
 #pragma unroll
-        for (int ks4 = 0; ks4 < 2 * S::NB; ++ks4) {  // 16 keys per step; rows ks4*16 + {0,8} + v_row share v_row's swizzle
-            const vec8 pf = as_vec8<vec8>(pfrag[ks4]);
-            const char FCK_LDS* vb = vt + ks4 * 16 * S::ROWB + v_rd;
+                for (int e = 0; e < 2; ++e) oacc[pr * 2 + e] = T::mfma32(as_vec8<vec8>(d[e]), pf, oacc[pr * 2 + e]);
+            } else {
+                const int t = m - kP;
+                const vec8 qv = as_vec8<vec8>(qf[t]);
 #pragma unroll
-            for (int dvb = 0; dvb < S::DVB; ++dvb) {
-                const int lc = dvb * 4 + v_c0;
-                const int coff = ((lc ^ v_swz<D>(v_row, lc)) << 4);
-                const u32x2_t lo4 = lds_read_tr16(vb + coff);
-                const u32x2_t hi4 = lds_read_tr16(vb + 8 * S::ROWB + coff);
-                const u32x4_t av = {lo4[0], lo4[1], hi4[0], hi4[1]};
-                oacc[dvb] = T::mfma32(as_vec8<vec8>(av), pf, oacc[dvb]);
+                for (int mbk = 0; mbk < 2; ++mbk) {
+                    if (t == 0) {
+                        f32x16_t z;
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) z[j] = 0.f;
+                        s[mbk] = T::mfma32(as_vec8<vec8>(d[mbk]), qv, z);
+                    } else {
+                        s[mbk] = T::mfma32(as_vec8<vec8>(d[mbk]), qv, s[mbk]);
+                    }
+                }
             }
+        };
+        fetch(0, bf[0]);
+        if (kSteps > 1) fetch(1, bf[1]);
+#pragma unroll
+        for (int m = 0; m < kSteps; ++m) {
+            if (m + 2 < kSteps) fetch(m + 2, bf[(m + 2) % 3]);
+            mma(m, bf[m % 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+
     // online softmax of local tile i: s -> pfrag
     auto softmax = [&](int i) __attribute__((always_inline)) {
         const int kb = (t_begin + i) * S::BN;
@@ -321,83 +362,40 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     };
 
     if (n > 0) {
-        // Three tiles are in flight from global memory: set (i % 3) holds (K_{i+1}, V_i) from step(i-3) until step(i).
-        Regs R0, R1, R2;
+        typedef std::integral_constant<int, 0> Keep0;
+        typedef std::integral_constant<int, 2 * S::LD> KeepPhase;  // the requests of one matrix phase
         if constexpr (kUniformPage) __syncthreads();  // page ids are in LDS
-        auto tile = [&](int i) __attribute__((always_inline)) { return min(i, n - 1); };  // clamp past-the-end requests
-        {
-            int64_t r[4] = {0, 0, 0, 0};
-            if constexpr (kUniformPage) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) r[t] = tile_row0(tile(t));
-            }
-            load_tile(kp, 0, r[0], R0.k);
-            store_k(0, R0);  // K_0 goes straight to LDS
-            load_tile(kp, tile(1), r[1], R0.k);
-            load_tile(vp, 0, r[0], R0.v);
-            load_tile(kp, tile(2), r[2], R1.k);
-            load_tile(vp, tile(1), r[1], R1.v);
-            load_tile(kp, tile(3), r[3], R2.k);
-            load_tile(vp, tile(2), r[2], R2.v);
-        }
+        request(kp, k_ring, 0, 0, cp_k);
+        request(vp, v_ring, 0, 0, cp_v);
+        request(kp, k_ring, 1, tile(1), cp_k);
+        wait_vm(Keep0{});
         __syncthreads();
-        // step(i, R), right after the matrix phase of tile i: write this thread's chunks of (K_{i+1}, V_i) from R and
-        // request (K_{i+4}, V_{i+3}) into the same registers.  Group 0 does this in phase 2i, group 1 in phase 2i+1;
-        // both halves are in LDS before phase 2i+2, the first one that reads them.
-        auto step = [&](int i, Regs& R, int64_t rk, int64_t rv) __attribute__((always_inline)) {
-            if (i + 1 < n) store_k(i + 1, R);
-            store_v(i, R);
-            load_tile(kp, tile(i + 4), rk, R.k);
-            load_tile(vp, tile(i + 3), rv, R.v);
-        };
-        // row bases of the tiles step(i) will request, looked up one matrix phase earlier
-        auto rows_for = [&](int i, int64_t& rk, int64_t& rv) __attribute__((always_inline)) {
-            rk = 0;
-            rv = 0;
-            if constexpr (kUniformPage) {
-                rv = tile_row0(tile(i + 3));
-                rk = tile_row0(tile(i + 4));
-            }
-        };
         if (group == 1) __syncthreads();  // skew: group 1 idles through phase 0
-        int64_t rk, rv;
-        rows_for(0, rk, rv);
-        qk(0);
-        step(0, R0, rk, rv);
+        // ring slots: c0 = i % kRing, c1 = (i + 1) % kRing, c2 = (i + 2) % kRing for the matrix phase M(i); it reads
+        // V from c0 and K from c1, and requests K_{i+3} into c0 and V_{i+2} into c2 (last read by M(i-1)).
+        int c0 = 2, c1 = 0, c2 = 1;  // i = -1
+        request(kp, k_ring, c0, tile(2), cp_k);
+        request(vp, v_ring, c2, tile(1), cp_v);
+        matrix(std::false_type{}, std::true_type{}, v_ring, k_ring + c1 * S::TILEB);
+        wait_vm(KeepPhase{});
         __syncthreads();
-        int i = 0;
-        while (true) {
-            if (i + 1 >= n) break;
+        for (int i = 0; i + 1 < n; ++i) {
             softmax(i);
             __syncthreads();
-            rows_for(i + 1, rk, rv);
-            pv(i);
-            qk(i + 1);
-            step(i + 1, R1, rk, rv);
+            const int c = c0;
+            c0 = c1;
+            c1 = c2;
+            c2 = c;
+            request(kp, k_ring, c0, tile(i + 3), cp_k);
+            request(vp, v_ring, c2, tile(i + 2), cp_v);
+            matrix(std::true_type{}, std::true_type{}, v_ring + c0 * S::TILEB, k_ring + c1 * S::TILEB);
+            wait_vm(KeepPhase{});
             __syncthreads();
-            ++i;
-            if (i + 1 >= n) break;
-            softmax(i);
-            __syncthreads();
-            rows_for(i + 1, rk, rv);
-            pv(i);
-            qk(i + 1);
-            step(i + 1, R2, rk, rv);
-            __syncthreads();
-            ++i;
-            if (i + 1 >= n) break;
-            softmax(i);
-            __syncthreads();
-            rows_for(i + 1, rk, rv);
-            pv(i);
-            qk(i + 1);
-            step(i + 1, R0, rk, rv);
-            __syncthreads();
-            ++i;
         }
         softmax(n - 1);
         __syncthreads();
-        pv(n - 1);
+        matrix(std::true_type{}, std::false_type{}, v_ring + c1 * S::TILEB, k_ring);
+        wait_vm(Keep0{});  // nothing may still be landing in LDS when the workgroup retires
         __syncthreads();
         if (group == 0) __syncthreads();  // both groups pass the same number of barriers
     }
@@ -424,7 +422,7 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
 {
     const int g = a.hq / a.hk, gx = (a.batch * a.hk + 7) / 8;
     const dim3 grid(8 * a.m_tiles * gx * g);
-    constexpr size_t lds = (size_t)4 * PPShape<D, BN>::TILEB + 8 * PPShape<D, BN>::KT * 1024 + kPrefillPageCache * 4;
+    constexpr size_t lds = (size_t)2 * PPShape<D, BN>::RING * PPShape<D, BN>::TILEB + kPrefillPageCache * 4;
     hipError_t e;
     if (uniform) {
         auto kern = prefill_pp_kernel<T, D, BN, true>;
