@@ -39,7 +39,7 @@ struct PPShape {
     static constexpr int CH = D / 8;    // 16-byte chunks per row
     static constexpr int TILEB = BN * ROWB;
     static constexpr int LD = TILEB / 1024 / 8;  // 1 KiB global->LDS instructions per wave and tile
-    static constexpr int RING = 3;               // LDS buffers per operand
+    static constexpr int RING = 4;               // LDS buffers per operand (a power of two)
     static_assert(TILEB % 8192 == 0, "a tile is split evenly over the 8 waves");
 };
 
@@ -173,33 +173,32 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         cp_v[u] = (D >= 128 ? (t ^ (((t >> 1) & 1) << 3)) : t) * 8;  // inverse of lc -> lc ^ v_swz(row, lc)
     }
 
-    // Page ids (uniform-page path): the pages of this workgroup's tiles are copied into LDS once, so the lookups of
-    // the main loop are LDS reads.  The host only selects this path when a sequence cannot have more than
-    // kPrefillPageCache tiles.
+    // First cache row of every tile (uniform-page path): computed once per workgroup into LDS, so the main loop needs
+    // one LDS read per tile and no table lookup.  The host only selects this path when a sequence cannot have more
+    // than kPrefillPageCache tiles.
     constexpr int kPageCache = kPrefillPageCache;
-    int FCK_LDS* page_lds = (int FCK_LDS*)(lds + 2 * kRing * S::TILEB);
-    auto page_index = [&](int key) __attribute__((always_inline)) {
-        return a.kv.page_shift >= 0 ? key >> a.kv.page_shift : key / a.kv.page_size;
-    };
+    int FCK_LDS* row_lds = (int FCK_LDS*)(lds + 2 * kRing * S::TILEB);
     if constexpr (kUniformPage) {
         if (ks.table != nullptr)
-            for (int i = tid; i < min(n, kPageCache); i += 512) page_lds[i] = ks.table[page_index((t_begin + i) * S::BN)];
+            for (int i = tid; i < min(n, kPageCache); i += 512) {
+                const int kb = (t_begin + i) * S::BN;
+                const int pi = a.kv.page_shift >= 0 ? kb >> a.kv.page_shift : kb / a.kv.page_size;
+                row_lds[i] = ks.table[pi] * a.kv.page_size + (kb - pi * a.kv.page_size);
+            }
     }
     auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t {
-        const int kb = (t_begin + i) * S::BN;
-        if (ks.table != nullptr) {
-            const int page = __builtin_amdgcn_readfirstlane(page_lds[i]);
-            return (int64_t)page * a.kv.page_size + (kb - page_index(kb) * a.kv.page_size);
-        }
-        return ks.base_row + kb;
+        if (ks.table != nullptr) return __builtin_amdgcn_readfirstlane(row_lds[i]);
+        return ks.base_row + (t_begin + i) * S::BN;
     };
     auto tile = [&](int i) __attribute__((always_inline)) { return min(i, n - 1); };  // requests past the end re-read the last tile
-    // request this wave's share of local tile i into ring buffer `slot` (wave-uniform)
-    auto request = [&](const uint16_t* base, char FCK_LDS* ring, int slot_, int i, const int (&cp_c)[S::LD]) __attribute__((always_inline)) {
-        const int kb = (t_begin + i) * S::BN;
-        const int room = last_key - kb;
+    // request this wave's share of local tile `want` into ring buffer want % kRing (past the last tile: that tile again)
+    auto request = [&](const uint16_t* base, char FCK_LDS* ring, int want, const int (&cp_c)[S::LD]) __attribute__((always_inline)) {
+        const int i = tile(want);
         int64_t row0 = 0;
         if constexpr (kUniformPage) row0 = tile_row0(i);
+        const int kb = (t_begin + i) * S::BN;
+        const int room = last_key - kb;
+        const int slot_ = want & (kRing - 1);
 #pragma unroll
         for (int u = 0; u < S::LD; ++u) {
             const int row = min(cp_row[u], room);  // rows past the last key repeat it (their scores are masked)
@@ -293,12 +292,17 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         };
         fetch(0, bf[0]);
         if (kSteps > 1) fetch(1, bf[1]);
+        // The wave in its matrix phase outranks the wave it shares the SIMD with (in its vector phase): at equal
+        // priority the vector-phase wave always has an instruction ready and wins the issue slot, the matrix pipe
+        // starves and the two phases run one after the other instead of side by side.
+        __builtin_amdgcn_s_setprio(3);
 #pragma unroll
         for (int m = 0; m < kSteps; ++m) {
             if (m + 2 < kSteps) fetch(m + 2, bf[(m + 2) % 3]);
             mma(m, bf[m % 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_s_setprio(0);
     };
 
     // online softmax of local tile i: s -> pfrag
@@ -363,38 +367,35 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
 
     if (n > 0) {
         typedef std::integral_constant<int, 0> Keep0;
-        typedef std::integral_constant<int, 2 * S::LD> KeepPhase;  // the requests of one matrix phase
-        if constexpr (kUniformPage) __syncthreads();  // page ids are in LDS
-        request(kp, k_ring, 0, 0, cp_k);
-        request(vp, v_ring, 0, 0, cp_v);
-        request(kp, k_ring, 1, tile(1), cp_k);
-        wait_vm(Keep0{});
+        typedef std::integral_constant<int, 2 * S::LD> KeepBatch;  // one batch = this wave's share of one K and one V tile
+        if constexpr (kUniformPage) __syncthreads();  // the row cache is in LDS
+        // Batch j = (K_{j+3}, V_{j+2}) is requested in the vector phase V(j), where the wave has issue slots to spare,
+        // and has landed when the wave leaves M(j+1); M(j+2) is the first phase that reads it.  Tile t lives in ring
+        // buffer t % kRing: while batch j is requested the other group may still read K_j and V_{j-1}, and K_{j+1},
+        // K_{j+2}, V_j, V_{j+1} are waiting or in flight, hence four buffers per operand.
+        request(kp, k_ring, 0, cp_k);
+        request(vp, v_ring, 0, cp_v);
+        request(kp, k_ring, 1, cp_k);
+        request(kp, k_ring, 2, cp_k);  // batch -1
+        request(vp, v_ring, 1, cp_v);
+        wait_vm(KeepBatch{});
         __syncthreads();
         if (group == 1) __syncthreads();  // skew: group 1 idles through phase 0
-        // ring slots: c0 = i % kRing, c1 = (i + 1) % kRing, c2 = (i + 2) % kRing for the matrix phase M(i); it reads
-        // V from c0 and K from c1, and requests K_{i+3} into c0 and V_{i+2} into c2 (last read by M(i-1)).
-        int c0 = 2, c1 = 0, c2 = 1;  // i = -1
-        request(kp, k_ring, c0, tile(2), cp_k);
-        request(vp, v_ring, c2, tile(1), cp_v);
-        matrix(std::false_type{}, std::true_type{}, v_ring, k_ring + c1 * S::TILEB);
-        wait_vm(KeepPhase{});
+        matrix(std::false_type{}, std::true_type{}, v_ring, k_ring);
         __syncthreads();
         for (int i = 0; i + 1 < n; ++i) {
+            request(kp, k_ring, i + 3, cp_k);
+            request(vp, v_ring, i + 2, cp_v);
             softmax(i);
             __syncthreads();
-            const int c = c0;
-            c0 = c1;
-            c1 = c2;
-            c2 = c;
-            request(kp, k_ring, c0, tile(i + 3), cp_k);
-            request(vp, v_ring, c2, tile(i + 2), cp_v);
-            matrix(std::true_type{}, std::true_type{}, v_ring + c0 * S::TILEB, k_ring + c1 * S::TILEB);
-            wait_vm(KeepPhase{});
+            matrix(std::true_type{}, std::true_type{}, v_ring + (i & (kRing - 1)) * S::TILEB,
+                   k_ring + ((i + 1) & (kRing - 1)) * S::TILEB);
+            wait_vm(KeepBatch{});
             __syncthreads();
         }
         softmax(n - 1);
         __syncthreads();
-        matrix(std::true_type{}, std::false_type{}, v_ring + c1 * S::TILEB, k_ring);
+        matrix(std::true_type{}, std::false_type{}, v_ring + ((n - 1) & (kRing - 1)) * S::TILEB, k_ring);
         wait_vm(Keep0{});  // nothing may still be landing in LDS when the workgroup retires
         __syncthreads();
         if (group == 0) __syncthreads();  // both groups pass the same number of barriers
