@@ -186,16 +186,24 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
                 row_lds[i] = ks.table[pi] * a.kv.page_size + (kb - pi * a.kv.page_size);
             }
     }
+    // Lane l keeps the first row of tile row_chunk * 64 + l in a register; a lookup is then a v_readlane, and LDS is
+    // read once per 64 tiles (an LDS read in every phase would queue behind the operand reads of the matrix phase).
+    int row_vec = 0, row_chunk = -1;
     auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t {
-        if (ks.table != nullptr) return __builtin_amdgcn_readfirstlane(row_lds[i]);
+        if (ks.table != nullptr) {
+            if ((i >> 6) != row_chunk) {
+                row_chunk = i >> 6;
+                row_vec = row_lds[min(row_chunk * 64 + lane, kPageCache - 1)];
+            }
+            return __builtin_amdgcn_readlane(row_vec, i & 63);
+        }
         return ks.base_row + (t_begin + i) * S::BN;
     };
     auto tile = [&](int i) __attribute__((always_inline)) { return min(i, n - 1); };  // requests past the end re-read the last tile
-    // request this wave's share of local tile `want` into ring buffer want % kRing (past the last tile: that tile again)
-    auto request = [&](const uint16_t* base, char FCK_LDS* ring, int want, const int (&cp_c)[S::LD]) __attribute__((always_inline)) {
+    // request this wave's share of local tile `want` into ring buffer want % kRing (past the last tile: that tile
+    // again); row0 = tile_row0(tile(want)) on the uniform-page path
+    auto request = [&](const uint16_t* base, char FCK_LDS* ring, int want, int64_t row0, const int (&cp_c)[S::LD]) __attribute__((always_inline)) {
         const int i = tile(want);
-        int64_t row0 = 0;
-        if constexpr (kUniformPage) row0 = tile_row0(i);
         const int kb = (t_begin + i) * S::BN;
         const int room = last_key - kb;
         const int slot_ = want & (kRing - 1);
@@ -373,19 +381,29 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         // and has landed when the wave leaves M(j+1); M(j+2) is the first phase that reads it.  Tile t lives in ring
         // buffer t % kRing: while batch j is requested the other group may still read K_j and V_{j-1}, and K_{j+1},
         // K_{j+2}, V_j, V_{j+1} are waiting or in flight, hence four buffers per operand.
-        request(kp, k_ring, 0, cp_k);
-        request(vp, v_ring, 0, cp_v);
-        request(kp, k_ring, 1, cp_k);
-        request(kp, k_ring, 2, cp_k);  // batch -1
-        request(vp, v_ring, 1, cp_v);
+        int64_t r0 = 0, r1 = 0, r2 = 0;
+        if constexpr (kUniformPage) {
+            r0 = tile_row0(0);
+            r1 = tile_row0(tile(1));
+            r2 = tile_row0(tile(2));
+        }
+        request(kp, k_ring, 0, r0, cp_k);
+        request(vp, v_ring, 0, r0, cp_v);
+        request(kp, k_ring, 1, r1, cp_k);
+        request(kp, k_ring, 2, r2, cp_k);  // batch -1
+        request(vp, v_ring, 1, r1, cp_v);
         wait_vm(KeepBatch{});
         __syncthreads();
         if (group == 1) __syncthreads();  // skew: group 1 idles through phase 0
         matrix(std::false_type{}, std::true_type{}, v_ring, k_ring);
         __syncthreads();
+        int64_t row_v = r2;  // first row of tile(i + 2): the tile whose K went out with the previous batch
         for (int i = 0; i + 1 < n; ++i) {
-            request(kp, k_ring, i + 3, cp_k);
-            request(vp, v_ring, i + 2, cp_v);
+            int64_t row_k = 0;
+            if constexpr (kUniformPage) row_k = tile_row0(tile(i + 3));
+            request(kp, k_ring, i + 3, row_k, cp_k);
+            request(vp, v_ring, i + 2, row_v, cp_v);
+            row_v = row_k;
             softmax(i);
             __syncthreads();
             matrix(std::true_type{}, std::true_type{}, v_ring + (i & (kRing - 1)) * S::TILEB,
