@@ -6,5 +6,6 @@ raises if it has not been built (`python -m flashck_amd.build`).
 from .utils import (FlashCKOperationType, get_available_operations, get_flashck_functions,  # noqa: F401
                     get_operation_function, is_available, register_flashck_functions)
 from . import ops  # noqa: F401
+from . import nn  # noqa: F401
 
 __version__ = "0.1.0"

@@ -23,8 +23,8 @@ from ...utils import FlashCKOperationType, register_flashck_functions
 __all__ = [
     "MASK_NONE", "MASK_TOP_LEFT", "MASK_BOTTOM_RIGHT", "MASK_GENERIC", "ROPE_NONE", "ROPE_INTERLEAVED",
     "ROPE_HALF_ROTATED", "fmha_fwd", "fmha_fwd_varlen", "fmha_fwd_splitkv", "fmha_fwd_splitkv_combine",
-    "fmha_fwd_appendkv", "fmha_batch_prefill", "fmha_fwd_pagedkv", "fmha_decode_paged", "num_splits_heuristic",
-    "splitkv_workspace",
+    "fmha_fwd_appendkv", "fmha_batch_prefill", "fmha_fwd_pagedkv", "fmha_decode_paged", "fmha_decode_step",
+    "DecodeWorkspace", "num_splits_heuristic", "splitkv_workspace",
 ]
 
 # GenericAttentionMaskEnum / RopeEnum, core/profiling/attention/fmha_library.h:81-87,195-200
@@ -315,6 +315,101 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
     return fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, out=out)
 
 
+class DecodeWorkspace:
+    """Buffers a decode step needs besides its inputs and outputs, kept between steps.
+
+    Holds the split-KV partials (o_acc, lse_acc) and the advanced key counts.  Buffers are only reallocated when a
+    step needs a larger one, so a serving loop with a fixed batch allocates on its first step only.
+    """
+
+    def __init__(self):
+        self._o_acc = None
+        self._lse_acc = None
+        self._seqlen = None
+        self._counts = None
+
+    @staticmethod
+    def _fit(buf, numel, dtype, device):
+        if buf is None or buf.numel() < numel or buf.dtype != dtype or buf.device != device:
+            buf = torch.empty(numel, dtype=dtype, device=device)
+        return buf
+
+    def partials(self, shape_batch, q_num_heads, num_splits, shape_seqlen_q, v_head_dim, device):
+        n_lse = shape_batch * q_num_heads * num_splits * shape_seqlen_q
+        self._o_acc = self._fit(self._o_acc, n_lse * v_head_dim, torch.float32, device)
+        self._lse_acc = self._fit(self._lse_acc, n_lse, torch.float32, device)
+        o_acc = self._o_acc[:n_lse * v_head_dim].view(shape_batch, q_num_heads, num_splits, shape_seqlen_q, v_head_dim)
+        lse_acc = self._lse_acc[:n_lse].view(shape_batch, q_num_heads, num_splits, shape_seqlen_q)
+        return o_acc, lse_acc
+
+    def lengths(self, batch, device):
+        self._seqlen = self._fit(self._seqlen, batch, torch.int32, device)
+        self._counts = self._fit(self._counts, batch, torch.int32, device)
+        return self._seqlen[:batch], self._counts[:batch]
+
+
+def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_knew=None,
+                     max_seqlen_knew: int = 0, rotary_cos=None, rotary_sin=None, rope_mode: int = ROPE_NONE,
+                     num_splits: int = 0, max_seqlen_k: int = 0, scale: float = 0.0, window_left: int = -1,
+                     workspace: Optional[DecodeWorkspace] = None, out=None):
+    """One serving step over a paged cache: append the new tokens, then attend from them.
+
+    The caller side of the split-KV path, FmhaKind::FwdAppendKV -> FwdSplitKV -> FwdSplitKVCombine
+    (core/profiling/attention/fmha_library.h:17-25), with the argument set of AttentionLayer
+    (core/module/layers/attention_layers/attention_layer.h:13-35):
+      1. knew is rotated and knew/vnew are written behind the seqlen_k[b] tokens of each sequence; q is rotated in
+         place at the same positions;
+      2. the split count comes from the CU count and the longest possible KV length unless num_splits is given;
+      3. split-KV forward over the seqlen_k[b] + n_b keys now in the cache - query i of a sequence sees keys up to
+         its own position (bottom-right causal; window_left >= 0 adds a sliding window) - and the LSE combine.
+    q/knew/vnew are [B, n, H, D] (n new tokens everywhere) or packed [total_new, H, D] with cu_seqlens_knew and
+    max_seqlen_knew.  Nothing is read back from the GPU, so a step only enqueues work on the current stream.
+
+    Returns (o, seqlen_k_new): o has q's shape (with Dv); seqlen_k_new = seqlen_k + n_b lives in the workspace and is
+    overwritten by the next step; seqlen_k itself is not modified.
+    """
+    packed = cu_seqlens_knew is not None
+    ws = workspace if workspace is not None else DecodeWorkspace()
+    B = seqlen_k.numel()
+    Hq, D = q.shape[-2], q.shape[-1]
+    Hk, Dv = k_cache.shape[2], v_cache.shape[3]
+    page = k_cache.shape[1]
+    if packed:
+        if max_seqlen_knew <= 0:
+            raise ValueError("packed new tokens need max_seqlen_knew")
+        n = int(max_seqlen_knew)
+    else:
+        if q.dim() != 4:
+            raise ValueError(f"q must be [B, n, Hq, D] without cu_seqlens_knew, got shape {tuple(q.shape)}")
+        n = q.shape[1]
+    fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, cu_seqlens_knew=cu_seqlens_knew, max_seqlen_knew=n,
+                      rotary_cos=rotary_cos, rotary_sin=rotary_sin, rope_mode=rope_mode, has_mask=True,
+                      block_table=block_table)
+    seqlen_new, counts = ws.lengths(B, seqlen_k.device)
+    if packed:
+        torch.sub(cu_seqlens_knew[1:], cu_seqlens_knew[:-1], out=counts)
+        torch.add(seqlen_k, counts, out=seqlen_new)
+    else:
+        torch.add(seqlen_k, n, out=seqlen_new)
+    if num_splits <= 0:
+        if max_seqlen_k <= 0:
+            max_seqlen_k = block_table.shape[1] * page  # what the block table can address
+        num_splits = num_splits_heuristic(B, Hq, Hk, n, max_seqlen_k, D)
+    # a lone new token sees every key: no mask needed unless a sliding window is asked for
+    if n == 1 and window_left < 0:
+        mask_type, window = MASK_NONE, (-1, -1)
+    else:
+        mask_type, window = MASK_BOTTOM_RIGHT, (int(window_left), 0)
+    shape_batch, shape_sq = (1, q.shape[0]) if packed else (B, n)
+    o_acc, lse_acc = ws.partials(shape_batch, Hq, num_splits, shape_sq, Dv, q.device)
+    fmha_fwd_splitkv(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_new, block_table=block_table,
+                     cu_seqlens_q=cu_seqlens_knew, max_seqlen_q=n if packed else 0, scale=scale, mask_type=mask_type,
+                     window=window, o_acc=o_acc, lse_acc=lse_acc)
+    o = fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_knew, max_seqlen_q=n if packed else 0,
+                                 out=out)
+    return o, seqlen_new
+
+
 register_flashck_functions(FlashCKOperationType.FMHA.value, {
     "forward": fmha_fwd,
     "forward_varlen": fmha_fwd_varlen,
@@ -324,4 +419,5 @@ register_flashck_functions(FlashCKOperationType.FMHA.value, {
     "batch_prefill": fmha_batch_prefill,
     "forward_pagedkv": fmha_fwd_pagedkv,
     "decode_paged": fmha_decode_paged,
+    "decode_step": fmha_decode_step,
 })

@@ -1,0 +1,73 @@
+"""The decode step (append -> split count -> split-KV -> combine) and the nn modules on the GPU, against the oracle."""
+import pytest
+import torch
+
+from flashck_amd import generators as gen
+from helpers import assert_bits_equal, assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _expected(orc, w, rope_mode, window_left=-1):
+    q, kc, vc = w["q"].clone(), w["k_cache"].clone(), w["v_cache"].clone()
+    orc.appendkv(q, kc, vc, w["knew"], w["vnew"], w["seqlen_k"], w["cu_seqlens_knew"], cos=w["rotary_cos"],
+                 sin=w["rotary_sin"], rope_mode=rope_mode, has_mask=True, block_table=w["block_table"])
+    sl = (w["seqlen_k"] + torch.tensor(w["new"], dtype=torch.int32)).contiguous()
+    o = orc.fmha_fwd(q, kc, vc, seqstart_q=w["cu_seqlens_knew"], seqlen_k=sl, block_table=w["block_table"],
+                     scale=w["scale"], mask_type=2, window=(window_left, 0))
+    return o, q, kc, vc, sl
+
+
+@pytest.mark.parametrize("num_splits", [0, 4])
+def test_decode_step_packed(fmha, orc, num_splits):
+    w = gen.workload_appendkv_decode(seed=71, batch=6, hq=8, hk=2, head_dim=128, min_len=0, max_len=700, max_new=9,
+                                     page_size=64)
+    ws = fmha.DecodeWorkspace()
+    q, kc, vc = dev(w["q"].clone()), dev(w["k_cache"].clone()), dev(w["v_cache"].clone())
+    sl = dev(w["seqlen_k"])
+    ro, rq, rkc, rvc, rsl = _expected(orc, w, 2)
+    for step in range(2):  # the second step reuses the workspace; inputs are restored so the result must repeat
+        q.copy_(w["q"])
+        kc.copy_(w["k_cache"])
+        vc.copy_(w["v_cache"])
+        o, sl_new = fmha.fmha_decode_step(q, dev(w["knew"]), dev(w["vnew"]), kc, vc, sl, dev(w["block_table"]),
+                                          cu_seqlens_knew=dev(w["cu_seqlens_knew"]), max_seqlen_knew=w["max_new"],
+                                          rotary_cos=dev(w["rotary_cos"]), rotary_sin=dev(w["rotary_sin"]), rope_mode=2,
+                                          num_splits=num_splits, scale=w["scale"], workspace=ws)
+        assert_bits_equal(q, rq, "rotated q")
+        assert_bits_equal(kc, rkc, "k cache")
+        assert_bits_equal(vc, rvc, "v cache")
+        assert torch.equal(sl_new.cpu(), rsl)
+        assert torch.equal(sl.cpu(), w["seqlen_k"])
+        assert_close(o, ro, 2e-2, f"decode step {step}")
+
+
+def test_paged_attention_module(fmha, orc):
+    from flashck_amd.nn import PagedAttention
+    # single new token per sequence, batch form, fp16
+    g = torch.Generator().manual_seed(72)
+    B, hq, hk, d, page = 5, 8, 4, 64, 16
+    lens = [0, 15, 16, 333, 64]
+    kv = gen.paged_kv(lens, hk, d, torch.float16, g, page, capacity=[l + 1 for l in lens])
+    q = gen.randn((B, 1, hq, d), torch.float16, g)
+    knew, vnew = gen.randn((B, 1, hk, d), torch.float16, g), gen.randn((B, 1, hk, d), torch.float16, g)
+    m = PagedAttention(hq, hk, d)
+    kc, vc = dev(kv["k_cache"].clone()), dev(kv["v_cache"].clone())
+    o, sl_new = m.decode_step(dev(q), dev(knew), dev(vnew), kc, vc, dev(kv["seqlen_k"]), dev(kv["block_table"]))
+    rkc, rvc = kv["k_cache"].clone(), kv["v_cache"].clone()
+    cu = torch.arange(B + 1, dtype=torch.int32)
+    orc.appendkv(None, rkc, rvc, knew.view(B, hk, d), vnew.view(B, hk, d), kv["seqlen_k"], cu, block_table=kv["block_table"])
+    assert_bits_equal(kc, rkc, "k cache")
+    assert_bits_equal(vc, rvc, "v cache")
+    ro = orc.fmha_fwd(q, rkc, rvc, seqlen_k=(kv["seqlen_k"] + 1).contiguous(), block_table=kv["block_table"])
+    assert_close(o, ro, 1e-2, "module decode step")
+    assert torch.equal(sl_new.cpu(), kv["seqlen_k"] + 1)
+
+
+def test_attention_module_dense(fmha, orc):
+    from flashck_amd.nn import Attention
+    w = gen.workload_dense_fp16()
+    m = Attention(w["q"].shape[2], w["k"].shape[2], w["q"].shape[3], scale=w["scale"])
+    o = m(dev(w["q"]), dev(w["k"]), dev(w["v"]))
+    ro = orc.fmha_fwd(w["q"], w["k"], w["v"], scale=w["scale"])
+    assert_close(o, ro, 1e-2, "Attention module, config 1")
