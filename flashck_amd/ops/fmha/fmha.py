@@ -18,13 +18,13 @@ from typing import Optional, Tuple
 import torch
 
 from ... import _lib
-from ...utils import FlashCKOperationType, register_flashck_functions
+from ...utils import FlashCKOperationType, register_flashck_functions, tuning
 
 __all__ = [
     "MASK_NONE", "MASK_TOP_LEFT", "MASK_BOTTOM_RIGHT", "MASK_GENERIC", "ROPE_NONE", "ROPE_INTERLEAVED",
     "ROPE_HALF_ROTATED", "fmha_fwd", "fmha_fwd_varlen", "fmha_fwd_splitkv", "fmha_fwd_splitkv_combine",
     "fmha_fwd_appendkv", "fmha_batch_prefill", "fmha_fwd_pagedkv", "fmha_decode_paged", "fmha_decode_step",
-    "DecodeWorkspace", "num_splits_heuristic", "splitkv_workspace",
+    "tune_decode_num_splits", "DecodeWorkspace", "num_splits_heuristic", "splitkv_workspace",
 ]
 
 # GenericAttentionMaskEnum / RopeEnum, core/profiling/attention/fmha_library.h:81-87,195-200
@@ -295,6 +295,14 @@ def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q
     return o
 
 
+def _auto_num_splits(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size, dtype) -> int:
+    """A tuned split count recorded for this class of problems if there is one, else the heuristic."""
+    return tuning.choose_num_splits(
+        lambda: num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim),
+        batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size,
+        "fp16" if dtype == torch.float16 else "bf16")
+
+
 def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits: int = 0, max_seqlen_k: int = 0,
                       cu_seqlens_q=None, max_seqlen_q: int = 0, scale: float = 0.0, mask_type: int = MASK_NONE,
                       window=(-1, -1), workspace=None, out=None) -> torch.Tensor:
@@ -307,12 +315,34 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
     if num_splits <= 0:
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * k_cache.shape[1]
-        num_splits = num_splits_heuristic(B, Hq, Hk, sq, max_seqlen_k, D)
+        num_splits = _auto_num_splits(B, Hq, Hk, sq, max_seqlen_k, D, k_cache.shape[1], q.dtype)
     o_acc, lse_acc = workspace if workspace is not None else (None, None)
     o_acc, lse_acc = fmha_fwd_splitkv(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_k, block_table=block_table,
                                       cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, scale=scale,
                                       mask_type=mask_type, window=window, o_acc=o_acc, lse_acc=lse_acc)
     return fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, out=out)
+
+
+def tune_decode_num_splits(q, k_cache, v_cache, seqlen_k, block_table, *, max_seqlen_k: int,
+                           candidates=(1, 2, 4, 8, 16, 32, 64), **kwargs) -> dict:
+    """Time `fmha_decode_paged` with each candidate split count on these tensors and record the fastest for the
+    problem class (see utils/tuning.py); later calls with num_splits = 0 on problems of that class use it.
+    Returns the record ({"num_splits", "latency_us", "tried_us", ...})."""
+    Hq, D = q.shape[-2], q.shape[-1]
+    Hk, page = k_cache.shape[2], k_cache.shape[1]
+    B = seqlen_k.numel()
+    sq = kwargs.get("max_seqlen_q", 0) or (q.shape[1] if q.dim() == 4 else 1)
+    problem = tuning.splitkv_problem(B, Hq, Hk, sq, max_seqlen_k, D, page, "fp16" if q.dtype == torch.float16 else "bf16")
+    ws = {}
+
+    def run(ns):
+        if ns not in ws:
+            shape_batch, shape_sq = (1, q.shape[0]) if q.dim() == 3 else (q.shape[0], q.shape[1])
+            ws[ns] = splitkv_workspace(shape_batch, Hq, shape_sq, v_cache.shape[3], ns, q.device)
+        fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, num_splits=ns, max_seqlen_k=max_seqlen_k,
+                          workspace=ws[ns], **kwargs)
+
+    return tuning.tune_num_splits(run, tuning.gpu_timer, candidates, problem)
 
 
 class DecodeWorkspace:
@@ -394,7 +424,7 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
     if num_splits <= 0:
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * page  # what the block table can address
-        num_splits = num_splits_heuristic(B, Hq, Hk, n, max_seqlen_k, D)
+        num_splits = _auto_num_splits(B, Hq, Hk, n, max_seqlen_k, D, page, q.dtype)
     # a lone new token sees every key: no mask needed unless a sliding window is asked for
     if n == 1 and window_left < 0:
         mask_type, window = MASK_NONE, (-1, -1)

@@ -71,3 +71,33 @@ def test_attention_module_dense(fmha, orc):
     o = m(dev(w["q"]), dev(w["k"]), dev(w["v"]))
     ro = orc.fmha_fwd(w["q"], w["k"], w["v"], scale=w["scale"])
     assert_close(o, ro, 1e-2, "Attention module, config 1")
+
+
+def test_tuned_split_count_is_recorded_and_used(fmha, orc, tmp_path):
+    import flashck_amd
+    from flashck_amd.utils import tuning
+    saved = {n: flashck_amd.get_flag_value(n) for n in ("FC_TUNING_DB_DIR", "FC_TUNING_NUM_COLD_ITERATION",
+                                                          "FC_TUNING_NUM_REPEATS", "FC_TUNING_MODE")}
+    old_default = tuning._default
+    try:
+        flashck_amd.set_flag_value("FC_TUNING_DB_DIR", str(tmp_path))
+        flashck_amd.set_flag_value("FC_TUNING_NUM_COLD_ITERATION", "2")
+        flashck_amd.set_flag_value("FC_TUNING_NUM_REPEATS", "5")
+        flashck_amd.set_flag_value("FC_TUNING_MODE", "2")
+        tuning._default = None
+        w = gen.workload_paged_decode(seed=73, batch=4, hq=16, hk=4, head_dim=128, min_len=900, max_len=2000, page_size=64)
+        q, kc, vc = dev(w["q"]), dev(w["k_cache"]), dev(w["v_cache"])
+        sl, bt = dev(w["seqlen_k"]), dev(w["block_table"])
+        rec = fmha.tune_decode_num_splits(q, kc, vc, sl, bt, max_seqlen_k=2048, candidates=(1, 2, 4, 8), scale=w["scale"])
+        assert rec["num_splits"] in (1, 2, 4, 8) and set(rec["tried_us"]) == {"1", "2", "4", "8"}
+        assert (tmp_path / tuning.FILE_NAME).exists()
+        prob = tuning.splitkv_problem(4, 16, 4, 1, 2048, 128, 64, "bf16")
+        assert tuning.default_cache().query(tuning.SPLITKV, prob)["num_splits"] == rec["num_splits"]
+        o = fmha.fmha_decode_paged(q, kc, vc, sl, bt, max_seqlen_k=2048, scale=w["scale"])  # num_splits = 0: the record
+        ro = orc.fmha_fwd(w["q"], w["k_cache"], w["v_cache"], seqlen_k=w["seqlen_k"], block_table=w["block_table"],
+                          scale=w["scale"])
+        assert_close(o, ro, 2e-2, "decode with the tuned split count")
+    finally:
+        for n, v in saved.items():
+            flashck_amd.set_flag_value(n, v)
+        tuning._default = old_default
