@@ -21,6 +21,12 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
 
+# HBM bytes one split-KV launch of the default workload moves, from two counter runs of this script
+# (`rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --no-extra --no-cpu --steps 20 --warmup 5`, then WRITE_SIZE):
+# 262,504.5 KiB fetched and 1,088 KiB written per dispatch, each scaled by what the same counter reads for a 512 MiB
+# device copy (`--workload copy`: FETCH_SIZE reads half the bytes copied -> x2.0, WRITE_SIZE reads them all -> x1.0).
+SPLITKV_DEFAULT_TRAFFIC_BYTES = int(262504.5 * 1024 * 2.0 + 1088 * 1024 * 1.0)
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -184,8 +190,10 @@ def main():
     if args.workload in ("splitkv", "paged_decode"):
         r = bench_decode(args, torch, fmha, gen, args.workload)
         value, unit, metric = r["gbs"], "GB/s", "paged-KV decode HBM GB/s (% of peak) + us/call; prefill TFLOP/s, MFMA util %"
+        default_shape = args.workload == "splitkv" and args.kv_len == 32768 and args.num_splits == 8 and not args.no_shuffle
+        traffic = SPLITKV_DEFAULT_TRAFFIC_BYTES if default_shape else None  # counters were only read for that shape
         roof = dict(bound="hbm", kernel="splitkv_decode_kernel", achieved=r["kernel_gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=r["kernel_gbs"] / HBM_PEAK_GBS, traffic=None, bytes_per_launch=r["bytes"],
+                    frac=r["kernel_gbs"] / HBM_PEAK_GBS, traffic=traffic, bytes_per_launch=r["bytes"],
                     avg_launch_us=r["kernel_ms"] * 1e3)
         extra["pct_of_hbm_peak"] = 100.0 * value / HBM_PEAK_GBS
         extra["us_per_call"] = r["ms_per_step"] * 1e3
@@ -197,7 +205,7 @@ def main():
         d = 128 if args.workload == "prefill" else 256
         r = bench_prefill(args, torch, fmha, gen, d, args.steps, args.warmup)
         value, unit, metric = r["tflops"], "TFLOP/s", "varlen causal prefill TFLOP/s (MFMA util %)"
-        roof = dict(bound="mfma", kernel="prefill_kernel", achieved=r["kernel_tflops"], peak=MFMA_BF16_PEAK_TFLOPS,
+        roof = dict(bound="mfma", kernel="prefill_pp_kernel" if d == 128 else "prefill_kernel", achieved=r["kernel_tflops"], peak=MFMA_BF16_PEAK_TFLOPS,
                     unit="TFLOP/s", frac=r["kernel_tflops"] / MFMA_BF16_PEAK_TFLOPS, traffic=None,
                     flops_per_launch=r["flops"], avg_launch_us=r["kernel_ms"] * 1e3)
         cpu = None
