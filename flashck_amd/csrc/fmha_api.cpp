@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <cstdlib>
 #include <cstdarg>
 #include <cstdio>
 #include <mutex>
@@ -254,6 +255,16 @@ int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* kne
     return launch_status(fck::launch_appendkv(a, dtype, (int)seqlen_knew, static_cast<hipStream_t>(stream)), "FmhaFwdAppendKV launch");
 }
 
+// The streaming (persistent-grid) prefill kernel is opt-in: FLASHCK_PREFILL_STREAM=1 in the environment of the process.
+static bool prefill_stream_enabled()
+{
+    static const bool on = [] {
+        const char* e = std::getenv("FLASHCK_PREFILL_STREAM");
+        return e != nullptr && e[0] == '1' && e[1] == 0;
+    }();
+    return on;
+}
+
 static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t q_max_seq_len, bool uniform, void* stream,
                           const char* what, int64_t max_keys_per_seq)
 {
@@ -264,6 +275,9 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t
     // head dim 256 take the 4-wave kernel (128 rows per workgroup).
     if (d <= 128 && q_max_seq_len > 128) {
         a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
+        const bool stream_uniform = uniform && max_keys_per_seq <= (int64_t)fck::kPrefillStreamRowCache * fck::kPrefillKeyTile;
+        if (prefill_stream_enabled() && stream_uniform && fck::prefill_stream_fits(a, cu_count()))
+            return launch_status(fck::launch_prefill_stream(a, (int)d, dtype, cu_count(), static_cast<hipStream_t>(stream)), what);
         return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, pp_uniform, static_cast<hipStream_t>(stream)), what);
     }
     a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);

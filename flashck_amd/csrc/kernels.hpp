@@ -74,4 +74,12 @@ constexpr int kPrefillKeyTile = 64;
 // 256-row workgroups (a.m_tiles counts 256-row tiles); head dims 64 and 128
 hipError_t launch_prefill_pingpong(const PrefillArgs& a, int d, int dtype, bool uniform_page, hipStream_t st);
 
+// Streaming (persistent) variant of the ping-pong kernel: one workgroup per CU walks a list of work items.  Limits:
+// first rows of at most kPrefillStreamRowCache key tiles per item are cached (uniform_page rule as above with this
+// count), and a workgroup's list holds at most kPrefillStreamMaxItems items (prefill_stream_fits).
+constexpr int kPrefillStreamRowCache = 2048;
+constexpr int kPrefillStreamMaxItems = 1024;
+bool prefill_stream_fits(const PrefillArgs& a, int num_cu);
+hipError_t launch_prefill_stream(const PrefillArgs& a, int d, int dtype, int num_cu, hipStream_t st);
+
 }  // namespace fck
