@@ -504,8 +504,8 @@ __global__ __launch_bounds__(512) void prefill_stream_kernel(const PrefillArgs a
             B = load_item(ii + 1);
             if (kc.buf == nxt) kc.chunk = -1;  // that half of the row cache changes hands
             if (vc.buf == nxt) vc.chunk = -1;
+            load_q(B, qnext);  // requested before the page-table reads below, so one wait covers both
             fill_rows(B, nxt);
-            load_q(B, qnext);
 #pragma unroll
             for (int t = 0; t < S::KT; ++t) asm volatile("" : "+v"(qnext[t]));  // have them landed here, not at the hand-off
         }
