@@ -199,7 +199,10 @@ def main():
         extra["us_per_call"] = r["ms_per_step"] * 1e3
         cpu = None
         if not args.no_cpu:
-            cpu = cpu_baseline_decode(r["w"], r["num_splits"], gen)
+            try:
+                cpu = cpu_baseline_decode(r["w"], r["num_splits"], gen)
+            except Exception as e:  # noqa: BLE001
+                cpu = dict(error=f"{type(e).__name__}: {e}")
         ms, name = r["ms_per_step"], r["name"]
     else:
         d = 128 if args.workload == "prefill" else 256
@@ -212,22 +215,34 @@ def main():
         ms, name = r["ms_per_step"], r["name"]
 
     if not args.no_extra and args.workload == "splitkv":
-        a2 = argparse.Namespace(**vars(args))
-        a2.steps, a2.warmup = max(20, args.steps // 2), 10
-        r2 = bench_decode(a2, torch, fmha, gen, "paged_decode")
-        extra["paged_decode"] = dict(workload=r2["name"], us_per_call=r2["ms_per_step"] * 1e3, gbs=r2["gbs"],
-                                     pct_of_hbm_peak=100 * r2["gbs"] / HBM_PEAK_GBS, kernel_us=r2["kernel_ms"] * 1e3,
-                                     bytes=r2["bytes"])
-        del r2
-        torch.cuda.empty_cache()
-        r4 = bench_appendkv(args, torch, fmha, gen, 100, 10)
-        extra["appendkv"] = dict(workload=r4["name"], us_per_call=r4["us_per_call"], bytes=r4["bytes"],
-                                 new_tokens=r4["new_tokens"])
-        for d in (128, 256):
+        # secondary workloads: a failure in one of them is reported in its place and does not cost the headline line
+        def secondary(name, fn):
+            try:
+                extra[name] = fn()
+            except Exception as e:  # noqa: BLE001
+                extra[name] = dict(error=f"{type(e).__name__}: {e}")
+            torch.cuda.empty_cache()
+
+        def paged():
+            a2 = argparse.Namespace(**vars(args))
+            a2.steps, a2.warmup = max(20, args.steps // 2), 10
+            r2 = bench_decode(a2, torch, fmha, gen, "paged_decode")
+            return dict(workload=r2["name"], us_per_call=r2["ms_per_step"] * 1e3, gbs=r2["gbs"],
+                        pct_of_hbm_peak=100 * r2["gbs"] / HBM_PEAK_GBS, kernel_us=r2["kernel_ms"] * 1e3, bytes=r2["bytes"])
+
+        def append():
+            r4 = bench_appendkv(args, torch, fmha, gen, 100, 10)
+            return dict(workload=r4["name"], us_per_call=r4["us_per_call"], bytes=r4["bytes"], new_tokens=r4["new_tokens"])
+
+        def prefill(d):
             r5 = bench_prefill(args, torch, fmha, gen, d, 10, 3)
-            extra[f"prefill_d{d}"] = dict(workload=r5["name"], ms_per_call=r5["ms_per_step"], tflops=r5["tflops"],
-                                          mfma_util_pct=100 * r5["tflops"] / MFMA_BF16_PEAK_TFLOPS, flops=r5["flops"],
-                                          kernel_ms=r5["kernel_ms"])
+            return dict(workload=r5["name"], ms_per_call=r5["ms_per_step"], tflops=r5["tflops"],
+                        mfma_util_pct=100 * r5["tflops"] / MFMA_BF16_PEAK_TFLOPS, flops=r5["flops"], kernel_ms=r5["kernel_ms"])
+
+        secondary("paged_decode", paged)
+        secondary("appendkv", append)
+        for d in (128, 256):
+            secondary(f"prefill_d{d}", lambda d=d: prefill(d))
 
     line = {
         "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
