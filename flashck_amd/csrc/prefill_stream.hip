@@ -299,20 +299,29 @@ __global__ __launch_bounds__(512) void prefill_stream_kernel(const PrefillArgs a
         const int t = pc ^ ((row & 3) << 1);
         cp_v[u] = (D >= 128 ? (t ^ (((t >> 1) & 1) << 3)) : t) * 8;  // inverse of lc -> lc ^ v_swz(row, lc)
     }
+    // byte offsets of this lane's chunks from the first row of a tile whose 64 rows all exist
+    uint32_t cp_koff[S::LD], cp_voff[S::LD];
+#pragma unroll
+    for (int u = 0; u < S::LD; ++u) {
+        cp_koff[u] = (uint32_t)(cp_row[u] * (int)row_stride + cp_k[u]) * 2u;
+        cp_voff[u] = (uint32_t)(cp_row[u] * (int)row_stride + cp_v[u]) * 2u;
+    }
     // request this wave's share of tile `tile` of item `it` (first cache row row0) into ring buffer `slot`
     auto request = [&](const uint16_t* base, char FCK_LDS* ring, int slot, const Item& it, int tile, int64_t row0,
-                       const int (&cp_c)[S::LD]) __attribute__((always_inline)) {
+                       const int (&cp_c)[S::LD], const uint32_t (&cp_off)[S::LD]) __attribute__((always_inline)) {
         const int room = it.sk_b - 1 - (it.t_begin + tile) * BN;
+        const bool whole = room >= BN - 1;  // every row of the tile exists (all tiles but the last of a sequence)
 #pragma unroll
         for (int u = 0; u < S::LD; ++u) {
-            const int row = min(cp_row[u], room);  // rows past the last key repeat it (their scores are masked)
             // Written as assembly on purpose: a load the compiler knows about makes it drain the whole load queue
             // before the next LDS read it cannot prove disjoint.  m0 carries the LDS address of the block and is
             // put back afterwards, since the compiler does not expect it to change.
             uint32_t m0_saved;
             const uint32_t dst = (uint32_t)(uintptr_t)(ring + slot * S::TILEB + (wave + 8 * u) * 1024);
             const uint16_t* tb = base + (row0 * row_stride + it.hkv * D);
-            const uint32_t off = (uint32_t)(row * (int)row_stride + cp_c[u]) * 2u;
+            uint32_t off = cp_off[u];
+            if (!whole)  // rows past the last key repeat it (their scores are masked)
+                off = (uint32_t)(min(cp_row[u], room) * (int)row_stride + cp_c[u]) * 2u;
             asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
                          : "=&s"(m0_saved)
                          : "s"(dst), "v"(off), "s"(tb)
@@ -512,22 +521,23 @@ __global__ __launch_bounds__(512) void prefill_stream_kernel(const PrefillArgs a
         const int n = A.n;
         const bool handoff = has_next && n >= 4 && B.n >= 3;
         // (item, tile, buffer of its first rows) a request for tile index `want` of the stream refers to
-        auto issue = [&](const uint16_t* base, char FCK_LDS* ring, int want, RowCache& c, const int (&cp_c)[S::LD]) __attribute__((always_inline)) {
+        auto issue = [&](const uint16_t* base, char FCK_LDS* ring, int want, RowCache& c, const int (&cp_c)[S::LD],
+                         const uint32_t (&cp_off)[S::LD]) __attribute__((always_inline)) {
             if (want < n) {
                 const int64_t row0 = tile_row0(A, cur, want, c);
-                request(base, ring, (pos + want) & (kRing - 1), A, want, row0, cp_c);
+                request(base, ring, (pos + want) & (kRing - 1), A, want, row0, cp_c, cp_off);
             } else if (handoff) {
                 const int64_t row0 = tile_row0(B, nxt, want - n, c);
-                request(base, ring, (pos + want) & (kRing - 1), B, want - n, row0, cp_c);
+                request(base, ring, (pos + want) & (kRing - 1), B, want - n, row0, cp_c, cp_off);
             }
         };
         if (n > 0) {
             if (!warm) {
-                issue(kp, k_ring, 0, kc, cp_k);
-                issue(vp, v_ring, 0, vc, cp_v);
-                issue(kp, k_ring, 1, kc, cp_k);
-                issue(kp, k_ring, 2, kc, cp_k);
-                issue(vp, v_ring, 1, vc, cp_v);
+                issue(kp, k_ring, 0, kc, cp_k, cp_koff);
+                issue(vp, v_ring, 0, vc, cp_v, cp_voff);
+                issue(kp, k_ring, 1, kc, cp_k, cp_koff);
+                issue(kp, k_ring, 2, kc, cp_k, cp_koff);
+                issue(vp, v_ring, 1, vc, cp_v, cp_voff);
                 if (n >= 3 || handoff)
                     wait_vm(KeepBatch{});
                 else
@@ -538,8 +548,8 @@ __global__ __launch_bounds__(512) void prefill_stream_kernel(const PrefillArgs a
                 __syncthreads();
             }
             for (int i = 0; i + 1 < n; ++i) {
-                issue(kp, k_ring, i + 3, kc, cp_k);
-                issue(vp, v_ring, i + 2, vc, cp_v);
+                issue(kp, k_ring, i + 3, kc, cp_k, cp_koff);
+                issue(vp, v_ring, i + 2, vc, cp_v, cp_voff);
                 softmax(i);
                 __syncthreads();
                 matrix(std::true_type{}, std::true_type{}, v_ring + ((pos + i) & (kRing - 1)) * S::TILEB,
@@ -551,8 +561,8 @@ __global__ __launch_bounds__(512) void prefill_stream_kernel(const PrefillArgs a
                 __syncthreads();
             }
             if (handoff) {
-                issue(kp, k_ring, n + 2, kc, cp_k);
-                issue(vp, v_ring, n + 1, vc, cp_v);
+                issue(kp, k_ring, n + 2, kc, cp_k, cp_koff);
+                issue(vp, v_ring, n + 1, vc, cp_v, cp_voff);
             }
             softmax(n - 1);
             __syncthreads();
