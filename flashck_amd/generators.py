@@ -140,10 +140,12 @@ def workload_appendkv_decode(seed=BASE_SEED + 4, batch=16, hq=32, hk=8, head_dim
 
 
 def workload_varlen_prefill(seed=BASE_SEED + 5, batch=16, hq=32, hk=8, head_dim=128, min_len=128, max_len=8192,
-                            page_size=128, dtype=torch.bfloat16):
-    """5: varlen causal batch prefill, sq = sk = L_b packed by cu_seqlens, K/V in a shuffled paged cache."""
+                            page_size=128, dtype=torch.bfloat16, lens=None):
+    """5: varlen causal batch prefill, sq = sk = L_b packed by cu_seqlens, K/V in a shuffled paged cache.
+    `lens` fixes the lengths instead of drawing them."""
     g = _gen(seed)
-    lens = randint_list(min_len, max_len, batch, g)
+    lens = list(lens) if lens is not None else randint_list(min_len, max_len, batch, g)
+    batch = len(lens)
     kv = paged_kv(lens, hk, head_dim, dtype, g, page_size)
     cu = torch.zeros(batch + 1, dtype=torch.int32)
     cu[1:] = torch.tensor(lens).cumsum(0)
