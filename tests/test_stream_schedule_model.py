@@ -181,3 +181,44 @@ def test_the_model_rejects_broken_schedules():
         with pytest.raises(AssertionError, match=what):
             for case in ([4, 4], [8, 3, 4, 9], [12, 12, 12], [5], [3, 8], [6, 1, 7], [9, 2]):
                 ns["check"](case)
+
+
+def _deal(total, nwx):
+    """Work-list dealing of the kernel: rank k of the valid slots goes to workgroup snake(k) at list position 2*round (+1)."""
+    lists = {w: {} for w in range(nwx)}
+    for k in range(total):
+        m = k % (2 * nwx)
+        for wgx in range(nwx):
+            which = 0 if m == wgx else (1 if m == 2 * nwx - 1 - wgx else -1)
+            if which >= 0:
+                lists[wgx][2 * (k // (2 * nwx)) + which] = k
+    counts = {}
+    for wgx in range(nwx):
+        rem = total % (2 * nwx)
+        counts[wgx] = 2 * (total // (2 * nwx)) + (1 if rem > wgx else 0) + (1 if rem > 2 * nwx - 1 - wgx else 0)
+    return lists, counts
+
+
+def test_work_list_dealing_is_a_partition_with_dense_ordered_lists():
+    for nwx in (1, 2, 3, 32):
+        for total in list(range(0, 4 * nwx + 3)) + [824, 1000]:
+            lists, counts = _deal(total, nwx)
+            seen = sorted(k for l in lists.values() for k in l.values())
+            assert seen == list(range(total)), (nwx, total)                    # every valid slot, exactly once
+            for wgx, l in lists.items():
+                assert sorted(l) == list(range(counts[wgx])), (nwx, total, wgx)  # positions 0..count-1, no holes
+                ranks = [l[p] for p in sorted(l)]
+                assert ranks == sorted(ranks)                                    # heaviest (lowest rank) first
+            assert max(counts.values()) - min(counts.values()) <= 2
+            assert max(counts.values()) <= total // nwx + 2                     # bound the launcher sizes the list with
+
+
+def test_work_list_balance_on_descending_costs():
+    # costs sorted in descending order (row tiles, heaviest first), as the slot order provides them
+    rng = random.Random(3)
+    for _ in range(20):
+        costs = sorted((rng.randint(1, 128) for _ in range(rng.randint(200, 2000))), reverse=True)
+        nwx = 32
+        lists, _ = _deal(len(costs), nwx)
+        loads = [sum(costs[k] for k in l.values()) for l in lists.values()]
+        assert max(loads) <= 1.05 * (sum(costs) / nwx) + 128
