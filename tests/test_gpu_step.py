@@ -101,3 +101,20 @@ def test_tuned_split_count_is_recorded_and_used(fmha, orc, tmp_path):
         for n, v in saved.items():
             flashck_amd.set_flag_value(n, v)
         tuning._default = old_default
+
+
+def test_page_size_one(fmha, orc):
+    """A page list with one token per page (the layout some serving stacks use): prefill and decode."""
+    w = gen.workload_varlen_prefill(seed=74, batch=4, hq=4, hk=2, head_dim=128, min_len=3, max_len=300, page_size=1)
+    o = fmha.fmha_batch_prefill(dev(w["q"]), dev(w["k_cache"]), dev(w["v_cache"]), dev(w["cu_seqlens_q"]), dev(w["kv_indptr"]),
+                                dev(w["kv_page_indices"]), dev(w["kv_last_page_lens"]), max_seqlen_q=w["max_seqlen_q"],
+                                scale=w["scale"])
+    ro = orc.fmha_fwd(w["q"], w["k_cache"], w["v_cache"], seqstart_q=w["cu_seqlens_q"], kv_indptr=w["kv_indptr"],
+                      kv_page_indices=w["kv_page_indices"], kv_last_page_lens=w["kv_last_page_lens"], scale=w["scale"],
+                      mask_type=2, window=(-1, 0))
+    assert_close(o, ro, 2e-2, "prefill, page size 1")
+    d = gen.workload_paged_decode(seed=75, batch=3, hq=8, hk=2, head_dim=128, min_len=1, max_len=500, page_size=1)
+    od = fmha.fmha_decode_paged(dev(d["q"]), dev(d["k_cache"]), dev(d["v_cache"]), dev(d["seqlen_k"]), dev(d["block_table"]),
+                                num_splits=3, scale=d["scale"])
+    rd = orc.fmha_fwd(d["q"], d["k_cache"], d["v_cache"], seqlen_k=d["seqlen_k"], block_table=d["block_table"], scale=d["scale"])
+    assert_close(od, rd, 2e-2, "decode, page size 1")
