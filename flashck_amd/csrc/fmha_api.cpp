@@ -255,13 +255,21 @@ int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* kne
     return launch_status(fck::launch_appendkv(a, dtype, (int)seqlen_knew, static_cast<hipStream_t>(stream)), "FmhaFwdAppendKV launch");
 }
 
-// The streaming (persistent-grid) prefill kernel is opt-in: FLASHCK_PREFILL_STREAM=1 in the environment of the process.
+// Two prefill kernels are opt-in, by a variable in the environment of the process (read once): the streaming
+// (persistent-grid) kernel with FLASHCK_PREFILL_STREAM=1, the direct-to-LDS head-dim-256 kernel with FLASHCK_PREFILL_DMA256=1.
+static bool env_is_one(const char* name)
+{
+    const char* e = std::getenv(name);
+    return e != nullptr && e[0] == '1' && e[1] == 0;
+}
 static bool prefill_stream_enabled()
 {
-    static const bool on = [] {
-        const char* e = std::getenv("FLASHCK_PREFILL_STREAM");
-        return e != nullptr && e[0] == '1' && e[1] == 0;
-    }();
+    static const bool on = env_is_one("FLASHCK_PREFILL_STREAM");
+    return on;
+}
+static bool prefill_dma256_enabled()
+{
+    static const bool on = env_is_one("FLASHCK_PREFILL_DMA256");
     return on;
 }
 
@@ -281,6 +289,8 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t
         return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, pp_uniform, static_cast<hipStream_t>(stream)), what);
     }
     a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
+    if (d == 256 && pp_uniform && prefill_dma256_enabled())
+        return launch_status(fck::launch_prefill_dma(a, (int)d, dtype, static_cast<hipStream_t>(stream)), what);
     return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
 }
 

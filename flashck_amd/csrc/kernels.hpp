@@ -79,6 +79,9 @@ hipError_t launch_prefill_pingpong(const PrefillArgs& a, int d, int dtype, bool 
 // count), and a workgroup's list holds at most kPrefillStreamMaxItems items (prefill_stream_fits).
 constexpr int kPrefillStreamRowCache = 2048;
 constexpr int kPrefillStreamMaxItems = 1024;
+// Head dim 256 with the K/V tiles sent global -> LDS directly (128-row workgroups; a.m_tiles counts 128-row tiles);
+// uniform pages with at most kPrefillPageCache key tiles per sequence.
+hipError_t launch_prefill_dma(const PrefillArgs& a, int d, int dtype, hipStream_t st);
 bool prefill_stream_fits(const PrefillArgs& a, int num_cu);
 hipError_t launch_prefill_stream(const PrefillArgs& a, int d, int dtype, int num_cu, hipStream_t st);
 

@@ -1,7 +1,9 @@
 """GPU parity of the streaming (persistent-grid) prefill kernel against the CPU oracle.
 
-The kernel is selected for a whole process by FLASHCK_PREFILL_STREAM=1, read once when the library takes its first
-prefill call.  It has not run on a GPU yet, so without that variable these tests are skipped; with it
+Two kernels are selected for a whole process by variables read once when the library takes its first prefill call:
+the streaming kernel by FLASHCK_PREFILL_STREAM=1 (first part of this file), the direct-to-LDS head-dim-256 kernel by
+FLASHCK_PREFILL_DMA256=1 (second part).  Neither has run on a GPU yet, so without its variable a test here is skipped;
+with it
 
     FLASHCK_PREFILL_STREAM=1 python -m pytest tests/test_gpu_stream.py tests/test_gpu_prefill.py -m gpu
 
@@ -15,9 +17,9 @@ import torch
 from flashck_amd import generators as gen
 from helpers import ATOL, assert_close, dev
 
-pytestmark = [pytest.mark.gpu,
-              pytest.mark.skipif(os.environ.get("FLASHCK_PREFILL_STREAM") != "1",
-                                 reason="the streaming prefill kernel has not run on a GPU yet; set FLASHCK_PREFILL_STREAM=1")]
+pytestmark = pytest.mark.gpu
+stream = pytest.mark.skipif(os.environ.get("FLASHCK_PREFILL_STREAM") != "1",
+                            reason="the streaming prefill kernel has not run on a GPU yet; set FLASHCK_PREFILL_STREAM=1")
 
 
 def _check(fmha, orc, w, dtype, what):
@@ -30,6 +32,7 @@ def _check(fmha, orc, w, dtype, what):
     assert_close(o, ro, ATOL[dtype], what)
 
 
+@stream
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("page", [64, 128])
@@ -40,6 +43,7 @@ def test_few_items_per_workgroup(fmha, orc, dtype, d, page):
     _check(fmha, orc, w, dtype, "one item per workgroup")
 
 
+@stream
 @pytest.mark.parametrize("d", [64, 128])
 def test_many_items_per_workgroup(fmha, orc, d):
     # 48 sequences x 16 heads x up to 5 row tiles on 256 workgroups: several items each, hand-offs between items of at
@@ -49,6 +53,7 @@ def test_many_items_per_workgroup(fmha, orc, d):
     _check(fmha, orc, w, torch.bfloat16, "several items per workgroup")
 
 
+@stream
 def test_short_and_long_sequences_mixed(fmha, orc):
     # one-tile and two-tile items (never handed off to) between long ones, one max_seqlen_q far above most lengths
     g = torch.Generator().manual_seed(170)
@@ -58,6 +63,7 @@ def test_short_and_long_sequences_mixed(fmha, orc):
     _check(fmha, orc, w, torch.bfloat16, "mixed lengths")
 
 
+@stream
 @pytest.mark.parametrize("mask", [(0, (-1, -1)), (2, (-1, 0)), (2, (100, 0)), (1, (-1, 0))])
 def test_dense_batch_mode_masks(fmha, orc, mask):
     # no page table: contiguous K/V, every mask kind, sliding window (row tiles that start past tile 0)
@@ -71,6 +77,7 @@ def test_dense_batch_mode_masks(fmha, orc, mask):
     assert_close(o, ro, 2e-2, "dense, streamed")
 
 
+@stream
 def test_repeated_launches_agree(fmha, orc):
     # the kernel keeps no state between launches: the same call twice gives the same bits
     w = gen.workload_varlen_prefill(seed=190, batch=20, hq=8, hk=2, head_dim=128, min_len=200, max_len=900, page_size=128)
@@ -78,3 +85,33 @@ def test_repeated_launches_agree(fmha, orc):
     o1 = fmha.fmha_batch_prefill(*args, max_seqlen_q=w["max_seqlen_q"], scale=w["scale"]).clone()
     o2 = fmha.fmha_batch_prefill(*args, max_seqlen_q=w["max_seqlen_q"], scale=w["scale"])
     assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# The direct-to-LDS head-dim-256 kernel (FLASHCK_PREFILL_DMA256=1): same status, same way to run it:
+#     FLASHCK_PREFILL_DMA256=1 python -m pytest tests/test_gpu_stream.py tests/test_gpu_prefill.py -m gpu -k "256 or dma"
+# ---------------------------------------------------------------------------------------------------------------------
+dma256 = pytest.mark.skipif(os.environ.get("FLASHCK_PREFILL_DMA256") != "1",
+                            reason="the direct-to-LDS head-dim-256 kernel has not run on a GPU yet; set FLASHCK_PREFILL_DMA256=1")
+
+
+@dma256
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("page", [64, 128])
+def test_dma256_paged(fmha, orc, dtype, page):
+    w = gen.workload_varlen_prefill(seed=250 + page, batch=6, hq=4, hk=2, head_dim=256, min_len=1, max_len=700,
+                                    page_size=page, dtype=dtype)
+    _check(fmha, orc, w, dtype, "head dim 256, direct to LDS")
+
+
+@dma256
+@pytest.mark.parametrize("mask", [(0, (-1, -1)), (2, (-1, 0)), (2, (90, 0)), (1, (-1, 0))])
+def test_dma256_dense_masks(fmha, orc, mask):
+    g = torch.Generator().manual_seed(260)
+    q = gen.randn((2, 300, 4, 256), torch.bfloat16, g)
+    k = gen.randn((2, 450, 2, 256), torch.bfloat16, g)
+    v = gen.randn((2, 450, 2, 256), torch.bfloat16, g)
+    mt, win = mask
+    o = fmha.fmha_fwd(dev(q), dev(k), dev(v), mask_type=mt, window=win)
+    ro = orc.fmha_fwd(q, k, v, mask_type=mt, window=win)
+    assert_close(o, ro, 2e-2, "dense, head dim 256")
