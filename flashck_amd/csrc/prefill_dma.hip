@@ -207,16 +207,21 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
         wait_all();
         __syncthreads();
     }
-    for (int i = 0; i < n; ++i) {
+    // One tile = head (request the next tile, S^T = K.Q^T, mask, row maxima), an occasional rescale, and the rest
+    // (exponentials, O^T += V^T.P^T, wait, barrier).  The rescale is the only place where vector instructions touch the
+    // output accumulator, so it lives outside the hot loop: with it inside, the compiler copies the whole accumulator
+    // out of the accumulation registers at the top of every iteration.
+    f32x16_t s[2];
+    float tmax = 0.f;
+    constexpr float kLazy = 8.f;
+    auto head = [&](int i) __attribute__((always_inline)) {
         const int buf = i & 1;
         const int kb = (t_begin + i) * BN;
         if (i + 1 < n) request(i + 1, buf ^ 1);  // the other buffer was last read before the barrier that ended tile i-1
 
         const char FCK_LDS* kt = lds + buf * S::TILEB;
-        const char FCK_LDS* vt = lds + (2 + buf) * S::TILEB;
 
         // ---- S^T = K . Q^T -------------------------------------------------------------------------------------
-        f32x16_t s[2];
 #pragma unroll
         for (int mbk = 0; mbk < 2; ++mbk) {
 #pragma unroll
@@ -230,7 +235,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
 
         // ---- online softmax (exp2 domain) ---------------------------------------------------------------------
         const bool need_mask = (kb < w_lo_max) || (kb + BN > w_hi_min);
-        float tmax = -INFINITY;
+        tmax = -INFINITY;
         if (need_mask) {
 #pragma unroll
             for (int mbk = 0; mbk < 2; ++mbk)
@@ -247,18 +252,10 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
             for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
         tmax = pair32_max(tmax);
         tmax *= a.scale_log2;  // scale > 0: max commutes with the scaling
-        // Lazy rescale: the reference m_run only moves when some row's maximum outgrows it by more than kLazy (log2
-        // units).  Softmax is shift invariant, so a stale reference is exact; it bounds the exponentials by 2^kLazy.
-        constexpr float kLazy = 8.f;
-        if (__builtin_amdgcn_ballot_w64(tmax > m_run + kLazy) != 0) {
-            const float m_new = fmaxf(m_run, tmax);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = fast_exp2(m_run - m_use);
-            m_run = m_new;
-            l_run *= alpha;
-#pragma unroll
-            for (int q = 0; q < S::DVB; ++q) oacc[q] *= alpha;
-        }
+    };
+    auto rest = [&](int i) __attribute__((always_inline)) {
+        const int buf = i & 1;
+        const char FCK_LDS* vt = lds + (2 + buf) * S::TILEB;
         const float m_ref = (m_run == -INFINITY) ? 0.f : m_run;
         float psum = 0.f;
 #pragma unroll
@@ -295,6 +292,32 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
 
         wait_all();       // this wave's share of tile i+1 has landed
         __syncthreads();  // ... and so has everyone's; nobody reads tile i any more
+    };
+    int i = 0;
+    while (i < n) {
+        bool rescale = false;
+        for (; i < n; ++i) {
+            head(i);
+            // Lazy rescale: the reference m_run only moves when some row's maximum outgrows it by more than kLazy (log2
+            // units).  Softmax is shift invariant, so a stale reference is exact; it bounds the exponentials by 2^kLazy.
+            if (__builtin_amdgcn_ballot_w64(tmax > m_run + kLazy) != 0) {
+                rescale = true;
+                break;
+            }
+            rest(i);
+        }
+        if (!rescale) break;
+        {
+            const float m_new = fmaxf(m_run, tmax);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = fast_exp2(m_run - m_use);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int q = 0; q < S::DVB; ++q) oacc[q] *= alpha;
+        }
+        rest(i);
+        ++i;
     }
 
     // ---- epilogue ----------------------------------------------------------------------------------------------------
