@@ -124,21 +124,20 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     const int64_t row_stride = (int64_t)a.hk * D;
 
     // global -> LDS assignment: wave w fills the 1 KiB blocks w, w+4, ... of a tile; lane l of an instruction lands at
-    // byte l*16 of its block, i.e. at (row, physical chunk) below, and fetches the logical chunk the swizzle maps there
-    int cp_row[S::LD];
-    uint32_t cp_koff[S::LD], cp_voff[S::LD], cp_kc[S::LD], cp_vc[S::LD];
-#pragma unroll
-    for (int u = 0; u < S::LD; ++u) {
-        const int off = (wave + 4 * u) * 1024 + lane * 16;
-        const int row = off / S::ROWB;
-        const int pc = (off % S::ROWB) >> 4;
-        cp_row[u] = row;
-        cp_kc[u] = (uint32_t)(pc ^ k_swz(row)) * 8u;
-        const int t = pc ^ ((row & 3) << 1);
-        cp_vc[u] = (uint32_t)(t ^ (((t >> 1) & 1) << 3)) * 8u;  // inverse of lc -> lc ^ v_swz(row, lc)
-        cp_koff[u] = ((uint32_t)(row * (int)row_stride) + cp_kc[u]) * 2u;
-        cp_voff[u] = ((uint32_t)(row * (int)row_stride) + cp_vc[u]) * 2u;
-    }
+    // byte l*16 of its block, i.e. at (row, physical chunk) below, and fetches the logical chunk the swizzle maps there.
+    // A 1 KiB block is two rows here, so block w + 4u holds rows cp_row0 + 8u (+1): the physical chunk is the same for
+    // every u, the K swizzle (row & 15) alternates with the parity of u and the V swizzle (row & 3) does not change.
+    // Three offset registers therefore serve all 16 instructions of a tile; the 8u rows go into the scalar base.
+    static_assert(S::ROWB == 512, "two rows per 1 KiB block");
+    const int cp_row0 = wave * 2 + (lane >> 5);
+    const int cp_pc = lane & 31;
+    const int cp_kc0 = (cp_pc ^ k_swz(cp_row0)) * 8;      // K chunk (element offset in the row), even u
+    const int cp_kc1 = (cp_pc ^ k_swz(cp_row0 + 8)) * 8;  // odd u
+    const int cp_t = cp_pc ^ ((cp_row0 & 3) << 1);
+    const int cp_vc = (cp_t ^ (((cp_t >> 1) & 1) << 3)) * 8;  // V chunk: inverse of lc -> lc ^ v_swz(row, lc)
+    const uint32_t cp_koff0 = (uint32_t)(cp_row0 * (int)row_stride + cp_kc0) * 2u;  // bytes from row 8u of the tile
+    const uint32_t cp_koff1 = (uint32_t)(cp_row0 * (int)row_stride + cp_kc1) * 2u;
+    const uint32_t cp_voff = (uint32_t)(cp_row0 * (int)row_stride + cp_vc) * 2u;
 
     // first cache row of every tile of this workgroup
     if (ks.table != nullptr) {
@@ -167,13 +166,18 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
         const int64_t tile_off = row0 * row_stride + hkv * D;
 #pragma unroll
         for (int kv = 0; kv < 2; ++kv) {
-            const uint16_t* tb = (kv == 0 ? kp : vp) + tile_off;
             char FCK_LDS* dst0 = lds + ((kv == 0 ? 0 : 2) + buf) * S::TILEB;
 #pragma unroll
             for (int u = 0; u < S::LD; ++u) {
-                uint32_t off = kv == 0 ? cp_koff[u] : cp_voff[u];
-                if (!whole)  // rows past the last key repeat it (their scores are masked)
-                    off = ((uint32_t)(min(cp_row[u], room) * (int)row_stride) + (kv == 0 ? cp_kc[u] : cp_vc[u])) * 2u;
+                const uint16_t* tb = (kv == 0 ? kp : vp) + tile_off;
+                uint32_t off;
+                if (whole) {
+                    tb += (int64_t)(8 * u) * row_stride;  // rows 8u .. of the tile, in the scalar base
+                    off = kv == 0 ? ((u & 1) ? cp_koff1 : cp_koff0) : cp_voff;
+                } else {  // rows past the last key repeat it (their scores are masked)
+                    const int row = min(cp_row0 + 8 * u, room);
+                    off = (uint32_t)(row * (int)row_stride + (kv == 0 ? ((u & 1) ? cp_kc1 : cp_kc0) : cp_vc)) * 2u;
+                }
                 // Written as assembly on purpose: a load the compiler knows about makes it drain the whole load queue
                 // before the next LDS read it cannot prove disjoint.  m0 carries the LDS address of the block and is put
                 // back afterwards, since the compiler does not expect it to change.
@@ -207,21 +211,16 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
         wait_all();
         __syncthreads();
     }
-    // One tile = head (request the next tile, S^T = K.Q^T, mask, row maxima), an occasional rescale, and the rest
-    // (exponentials, O^T += V^T.P^T, wait, barrier).  The rescale is the only place where vector instructions touch the
-    // output accumulator, so it lives outside the hot loop: with it inside, the compiler copies the whole accumulator
-    // out of the accumulation registers at the top of every iteration.
-    f32x16_t s[2];
-    float tmax = 0.f;
-    constexpr float kLazy = 8.f;
-    auto head = [&](int i) __attribute__((always_inline)) {
+    for (int i = 0; i < n; ++i) {
         const int buf = i & 1;
         const int kb = (t_begin + i) * BN;
         if (i + 1 < n) request(i + 1, buf ^ 1);  // the other buffer was last read before the barrier that ended tile i-1
 
         const char FCK_LDS* kt = lds + buf * S::TILEB;
+        const char FCK_LDS* vt = lds + (2 + buf) * S::TILEB;
 
         // ---- S^T = K . Q^T -------------------------------------------------------------------------------------
+        f32x16_t s[2];
 #pragma unroll
         for (int mbk = 0; mbk < 2; ++mbk) {
 #pragma unroll
@@ -235,7 +234,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
 
         // ---- online softmax (exp2 domain) ---------------------------------------------------------------------
         const bool need_mask = (kb < w_lo_max) || (kb + BN > w_hi_min);
-        tmax = -INFINITY;
+        float tmax = -INFINITY;
         if (need_mask) {
 #pragma unroll
             for (int mbk = 0; mbk < 2; ++mbk)
@@ -252,10 +251,28 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
             for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
         tmax = pair32_max(tmax);
         tmax *= a.scale_log2;  // scale > 0: max commutes with the scaling
-    };
-    auto rest = [&](int i) __attribute__((always_inline)) {
-        const int buf = i & 1;
-        const char FCK_LDS* vt = lds + (2 + buf) * S::TILEB;
+        // Lazy rescale: the reference m_run only moves when some row's maximum outgrows it by more than kLazy (log2
+        // units).  Softmax is shift invariant, so a stale reference is exact; it bounds the exponentials by 2^kLazy.
+        constexpr float kLazy = 8.f;
+        if (__builtin_amdgcn_ballot_w64(tmax > m_run + kLazy) != 0) {
+            const float m_new = fmaxf(m_run, tmax);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = fast_exp2(m_run - m_use);
+            m_run = m_new;
+            l_run *= alpha;
+            // The output accumulator lives in the accumulation half of the register file (the MFMAs update it there).
+            // It is scaled through explicit accumulator reads and writes inside this branch: a plain `oacc[q] *= alpha`
+            // makes the compiler copy all of it into vector registers at the top of every iteration.
+#pragma unroll
+            for (int q = 0; q < S::DVB; ++q)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    float x;
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(oacc[q][j]));
+                    x *= alpha;
+                    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(oacc[q][j]) : "v"(x));
+                }
+        }
         const float m_ref = (m_run == -INFINITY) ? 0.f : m_run;
         float psum = 0.f;
 #pragma unroll
@@ -292,32 +309,6 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
 
         wait_all();       // this wave's share of tile i+1 has landed
         __syncthreads();  // ... and so has everyone's; nobody reads tile i any more
-    };
-    int i = 0;
-    while (i < n) {
-        bool rescale = false;
-        for (; i < n; ++i) {
-            head(i);
-            // Lazy rescale: the reference m_run only moves when some row's maximum outgrows it by more than kLazy (log2
-            // units).  Softmax is shift invariant, so a stale reference is exact; it bounds the exponentials by 2^kLazy.
-            if (__builtin_amdgcn_ballot_w64(tmax > m_run + kLazy) != 0) {
-                rescale = true;
-                break;
-            }
-            rest(i);
-        }
-        if (!rescale) break;
-        {
-            const float m_new = fmaxf(m_run, tmax);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = fast_exp2(m_run - m_use);
-            m_run = m_new;
-            l_run *= alpha;
-#pragma unroll
-            for (int q = 0; q < S::DVB; ++q) oacc[q] *= alpha;
-        }
-        rest(i);
-        ++i;
     }
 
     // ---- epilogue ----------------------------------------------------------------------------------------------------
