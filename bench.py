@@ -41,24 +41,43 @@ def parse():
     ap.add_argument("--kv-len", type=int, default=32768, help="KV length of the split-KV workload (study runs only)")
     ap.add_argument("--no-shuffle", action="store_true", help="identity page order (study runs only)")
     ap.add_argument("--num-splits", type=int, default=8, help="split count of the split-KV workload (study runs only)")
+    ap.add_argument("--decode-path", default="two-launch", choices=["two-launch", "fused"],
+                    help="two-launch: split-KV + combine kernels with a caller-owned workspace; fused: one launch "
+                         "(--num-splits 0 lets the library choose the key ranges)")
     return ap.parse_args()
 
 
 def time_steps(fn, steps, warmup, torch, kernel_events=False):
-    """Runs fn(step, ev) warmup + steps times; returns (wall seconds for `steps`, avg ms between event pairs)."""
+    """Runs fn(step, ev) warmup + steps times.  Returns (wall seconds for `steps`, avg ms per launch by HIP events).
+
+    kernel_events = "region": one event pair on the launch stream brackets the whole timed region (for steps that are
+    a single launch: the average it gives includes the gaps between launches).  kernel_events = True: the timed region
+    carries no events; the same steps are then run once more with an event pair around the kernel of every step.
+    """
     for i in range(warmup):
         fn(i, None)
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)] \
-        if kernel_events else [None] * steps
+    region = kernel_events == "region"
+    if region:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    if region:
+        e0.record()
     for i in range(steps):
-        fn(warmup + i, evs[i])
+        fn(warmup + i, None)
+    if region:
+        e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     kern_ms = None
-    if kernel_events:
+    if region:
+        kern_ms = e0.elapsed_time(e1) / steps
+    elif kernel_events:
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i in range(steps):
+            fn(warmup + steps + i, evs[i])
+        torch.cuda.synchronize()
         kern_ms = sum(a.elapsed_time(b) for a, b in evs) / steps
     return wall, kern_ms
 
@@ -67,11 +86,20 @@ def bench_decode(args, torch, fmha, gen, which):
     if which == "splitkv":
         w = gen.workload_splitkv_decode(kv_len=args.kv_len, num_splits=args.num_splits, shuffle=not args.no_shuffle)
         ns = w["num_splits"]
-        name = f"split-KV long-context decode: B=4 q=1 Hq64/Hk8 D128 L={args.kv_len} P=128 ns={ns} + combine (bf16)"
+        if getattr(args, "decode_path", "two-launch") == "fused":
+            ns = args.num_splits
+            name = (f"split-KV long-context decode: B=4 q=1 Hq64/Hk8 D128 L={args.kv_len} P=128, one fused launch, "
+                    f"ns={ns if ns else 'library-chosen'} (bf16)")
+        else:
+            name = f"split-KV long-context decode: B=4 q=1 Hq64/Hk8 D128 L={args.kv_len} P=128 ns={ns} + combine (bf16)"
     else:
         w = gen.workload_paged_decode()
-        ns = fmha.num_splits_heuristic(32, 32, 8, 1, max(w["lens"]), 128)
-        name = f"paged-KV decode: B=32 q=1 Hq32/Hk8 D128 L~U[512,4096] P=128 ns={ns} + combine (bf16)"
+        if getattr(args, "decode_path", "two-launch") == "fused":
+            ns = 0
+            name = "paged-KV decode: B=32 q=1 Hq32/Hk8 D128 L~U[512,4096] P=128, one fused launch, library-chosen ranges (bf16)"
+        else:
+            ns = fmha.num_splits_heuristic(32, 32, 8, 1, max(w["lens"]), 128)
+            name = f"paged-KV decode: B=32 q=1 Hq32/Hk8 D128 L~U[512,4096] P=128 ns={ns} + combine (bf16)"
     B, _, Hq, D = w["q"].shape
     Hk = w["k_cache"].shape[2]
     dev = "cuda"
@@ -80,19 +108,25 @@ def bench_decode(args, torch, fmha, gen, which):
     pools = [(w["k_cache"].to(dev), w["v_cache"].to(dev))]
     for _ in range(args.copies - 1):
         pools.append((pools[0][0].clone(), pools[0][1].clone()))
-    o_acc, lse_acc = fmha.splitkv_workspace(B, Hq, 1, D, ns, dev)
+    o_acc, lse_acc = fmha.splitkv_workspace(B, Hq, 1, D, max(ns, 1), dev)
     o = torch.empty(B, 1, Hq, D, dtype=q.dtype, device=dev)
+
+    fused = getattr(args, "decode_path", "two-launch") == "fused"
 
     def step(i, ev):
         kc, vc = pools[i % len(pools)]
         if ev is not None:
             ev[0].record()
-        fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc)
+        if fused:
+            raise SystemExit("this build has no fused decode entry point")
+        else:
+            fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc)
         if ev is not None:
             ev[1].record()
-        fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, out=o)
+        if not fused:
+            fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, out=o)
 
-    wall, kern_ms = time_steps(step, args.steps, args.warmup, torch, kernel_events=True)
+    wall, kern_ms = time_steps(step, args.steps, args.warmup, torch, kernel_events="region" if fused else True)
     nbytes = gen.decode_bytes(w["lens"], [1] * B, Hq, Hk, D, D, 128)
     flops = gen.decode_flops(w["lens"], [1] * B, Hq, D, D)
     ms = wall / args.steps * 1e3

@@ -16,6 +16,7 @@ _vp, _i64, _i32, _u32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, c
 SIGNATURES = {
     "fck_last_error": (ctypes.c_char_p, []),
     "fck_fmha_version": (ctypes.c_char_p, []),
+    "fck_fmha_last_kernel": (ctypes.c_char_p, []),
     "fck_fmha_fwd": (ctypes.c_int, [_vp] * 8 + [_i64] * 8 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_fwd_splitkv": (ctypes.c_int, [_vp] * 11 + [_i64] * 11 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_fwd_splitkv_combine": (ctypes.c_int, [_vp] * 4 + [_i64] * 6 + [_i32, _vp]),

@@ -45,6 +45,11 @@ struct BF16 {
     {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    // 16x16x16: 4 packed elements per operand (for 16-key tiles)
+    static __device__ __forceinline__ f32x4_t mfma16k16(u32x2_t a, u32x2_t b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+    }
 };
 
 struct FP16 {
@@ -67,6 +72,10 @@ struct FP16 {
     static __device__ __forceinline__ f32x16_t mfma32(vec8 a, vec8 b, f32x16_t c)
     {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4_t mfma16k16(u32x2_t a, u32x2_t b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
     }
 };
 
@@ -134,6 +143,58 @@ __device__ __forceinline__ float quad16_sum(float x)
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// LSE combine of the split-KV partials of one output row, 4 columns from column c on:
+//   LSE = logsumexp_s lse_acc[s];  O = sum_s exp(lse_acc[s] - LSE) * o_acc[s]
+// (ck_tile/ops/fmha/pipeline/block_fmha_fwd_splitkv_combine_pipeline.hpp:150-316), evaluated as
+// O = (sum_s e^(lse_s - m) o_s) / (sum_s e^(lse_s - m)) with a running maximum m over batches of kCombineBatch splits, so
+// that all loads of a batch are in flight together: the work is a chain of memory round trips, not arithmetic.
+// w0 is the workspace row of split 0 and `step` the distance to the next split's row; rows whose splits are all empty
+// (-inf) give zeros; a single split is passed through unchanged.  Shared by the combine kernel and by the fused tail of
+// the split-KV kernel, so both produce the same bits.
+constexpr int kCombineBatch = 16;
+
+template <int DV>
+__device__ __forceinline__ f32x4_t combine_splits(const float* lse_acc, const float* o_acc, int64_t w0, int64_t step, int ns, int c)
+{
+    float m_run = -INFINITY, sum = 0.f;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < ns; s0 += kCombineBatch) {
+        float l[kCombineBatch];
+        f32x4_t v[kCombineBatch];
+#pragma unroll
+        for (int j = 0; j < kCombineBatch; ++j) {
+            const bool ok = s0 + j < ns;
+            const int64_t w = w0 + (ok ? s0 + j : s0) * step;  // out-of-range slots re-read a valid one and are dropped
+            const float lj = lse_acc[w];
+            l[j] = ok ? lj : -INFINITY;
+            v[j] = *reinterpret_cast<const f32x4_t*>(o_acc + w * DV + c);
+        }
+        float mb = l[0];
+#pragma unroll
+        for (int j = 1; j < kCombineBatch; ++j) mb = fmaxf(mb, l[j]);
+        const float m_new = fmaxf(m_run, mb);
+        if (m_new == -INFINITY) continue;
+        const float keep = __expf(m_run - m_new);  // 0 for the first non-empty batch
+        sum *= keep;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[k] *= keep;
+#pragma unroll
+        for (int j = 0; j < kCombineBatch; ++j) {
+            const float wgt = __expf(l[j] - m_new);
+            sum += wgt;
+            if (wgt != 0.f) {  // an empty split's partial row may hold anything
+#pragma unroll
+                for (int k = 0; k < 4; ++k) acc[k] = __builtin_fmaf(wgt, v[j][k], acc[k]);
+            }
+        }
+        m_run = m_new;
+    }
+    if (sum == 0.f) return f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (ns == 1) return acc;  // weight exactly 1
+    const float inv = 1.f / sum;
+    return f32x4_t{acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
+}
 
 // Visible key range [lo, hi) of query row i: GenericAttentionMask::IsOutOfBound,
 // ck_tile/ops/fmha/block/block_masking.hpp:359-373 with (y, x) from
@@ -212,7 +273,9 @@ __device__ __forceinline__ KvSeq kv_seq(const KvAddr& a, int b)
         const int s0 = a.seqstart_k[b];
         s.table = nullptr;
         s.base_row = s0;
-        s.len = a.seqstart_k[b + 1] - s0;
+        // packed K/V with padding: the logical length comes from seqlen_k_ptr when it is given
+        // (ck_tile/ops/fmha/kernel/fmha_fwd_splitkv_kernel.hpp:648-650)
+        s.len = a.seqlen_k_ptr ? a.seqlen_k_ptr[b] : a.seqstart_k[b + 1] - s0;
     } else if (a.mode == 2) {
         s.table = a.block_table + (int64_t)b * a.block_table_stride;
         s.base_row = 0;

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <climits>
 #include <cmath>
 #include <cstdlib>
 #include <cstdarg>
@@ -15,6 +16,7 @@
 namespace {
 
 thread_local char g_err[512] = "";
+thread_local const char* g_kernel = "";  // kernel family of the calling thread's last launch
 
 int fail(int code, const char* fmt, ...)
 {
@@ -78,7 +80,9 @@ extern "C" {
 
 const char* fck_last_error(void) { return g_err; }
 
-const char* fck_fmha_version(void) { return "flashck-fmha-gfx950 0.1"; }
+const char* fck_fmha_version(void) { return "flashck-fmha-gfx950 0.2"; }
+
+const char* fck_fmha_last_kernel(void) { return g_kernel; }
 
 size_t fck_fmha_splitkv_workspace_bytes(int64_t shape_batch, int64_t hq, int64_t shape_sq, int64_t dv, int64_t num_splits)
 {
@@ -108,32 +112,30 @@ int fck_fmha_num_splits_heuristic(int64_t batch, int64_t hq, int64_t hk, int64_t
     return (int)ns;
 }
 
-int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v, const void* bias, void* lse_acc, void* o_acc,
-                         const int32_t* seqstart_q, const int32_t* seqstart_k, const int32_t* seqlen_k_ptr,
+// Validation and argument block shared by the split-KV entry points (everything but the workspace / output pointers).
+static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, const void* q, const void* k, const void* v,
+                         const void* bias, const int32_t* seqstart_q, const int32_t* seqstart_k, const int32_t* seqlen_k_ptr,
                          const int32_t* block_table, const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
                          int64_t seqlen_k, int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len,
                          int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size, float scale,
-                         int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream)
+                         int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype)
 {
-    g_err[0] = 0;
     if (int rc = check_common(batch, hq, hk, d, dv, dtype, bias)) return rc;
     if (int rc = check_mask(mask_type)) return rc;
-    if (!q || !k || !v || !lse_acc || !o_acc) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v, lse_acc and o_acc must not be null");
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o_acc))
-        return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v and o_acc must be 16-byte aligned");
+    if (!q || !k || !v) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k and v must not be null");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k and v must be 16-byte aligned");
     if (num_splits < 1 || num_splits > 128) return fail(FCK_ERR_INVALID_ARGUMENT, "num_splits %ld out of range [1,128]", (long)num_splits);
     if (!(scale > 0.f) || !std::isfinite(scale)) return fail(FCK_ERR_INVALID_ARGUMENT, "scale must be positive and finite");
     const bool group = seqstart_q != nullptr;
     if (!group && seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "seqlen_q must be positive in batch mode");
+    if (group && seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "group mode: seqlen_q must carry total_q (workspace row count)");
     if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
     if (q_max_seq_len <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_max_seq_len must be positive");
 
-    fck::SplitKvArgs a{};
+    a = fck::SplitKvArgs{};
     a.q = q;
     a.k = k;
     a.v = v;
-    a.o_acc = static_cast<float*>(o_acc);
-    a.lse_acc = static_cast<float*>(lse_acc);
     a.seqstart_q = seqstart_q;
     a.batch = (int32_t)batch;
     a.sq = (int32_t)seqlen_q;
@@ -145,9 +147,8 @@ int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v, const void
     a.mask_type = mask_type;
     a.window_left = window_left;
     a.window_right = window_right;
-    if (group && seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "group mode: seqlen_q must carry total_q (workspace row count)");
 
-    bool uniform = true;
+    uniform = true;
     fck::KvAddr& kv = a.kv;
     kv.seqlen_k_ptr = seqlen_k_ptr;
     kv.cache_batch_idx = cache_batch_idx;
@@ -171,8 +172,31 @@ int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v, const void
         kv.mode = 0;
         kv.seqlen_k = (int32_t)seqlen_k;
     }
-    const int rows_max = (int)(q_max_seq_len * (hq / hk));
-    return launch_status(fck::launch_splitkv_decode(a, (int)d, dtype, rows_max, uniform, static_cast<hipStream_t>(stream)),
+    rows_max = (int)(q_max_seq_len * (hq / hk));
+    return FCK_OK;
+}
+
+int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v, const void* bias, void* lse_acc, void* o_acc,
+                         const int32_t* seqstart_q, const int32_t* seqstart_k, const int32_t* seqlen_k_ptr,
+                         const int32_t* block_table, const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
+                         int64_t seqlen_k, int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len,
+                         int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size, float scale,
+                         int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream)
+{
+    g_err[0] = 0;
+    fck::SplitKvArgs a;
+    bool uniform;
+    int rows_max;
+    if (int rc = splitkv_setup(a, uniform, rows_max, q, k, v, bias, seqstart_q, seqstart_k, seqlen_k_ptr, block_table,
+                               cache_batch_idx, batch, seqlen_q, seqlen_k, hq, hk, d, dv, q_max_seq_len, num_splits,
+                               max_num_page_blocks, page_block_size, scale, window_left, window_right, mask_type, dtype))
+        return rc;
+    if (!lse_acc || !o_acc) return fail(FCK_ERR_INVALID_ARGUMENT, "lse_acc and o_acc must not be null");
+    if (!aligned16(o_acc)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_acc must be 16-byte aligned");
+    a.o_acc = static_cast<float*>(o_acc);
+    a.lse_acc = static_cast<float*>(lse_acc);
+    g_kernel = uniform ? "splitkv_decode_kernel<uniform_page>" : "splitkv_decode_kernel<row_lookup>";
+    return launch_status(fck::launch_splitkv_decode(a, (int)d, dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
                          "FmhaFwdSplitKV launch");
 }
 
@@ -255,42 +279,22 @@ int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* kne
     return launch_status(fck::launch_appendkv(a, dtype, (int)seqlen_knew, static_cast<hipStream_t>(stream)), "FmhaFwdAppendKV launch");
 }
 
-// Two prefill kernels are opt-in, by a variable in the environment of the process (read once): the streaming
-// (persistent-grid) kernel with FLASHCK_PREFILL_STREAM=1, the direct-to-LDS head-dim-256 kernel with FLASHCK_PREFILL_DMA256=1.
-static bool env_is_one(const char* name)
-{
-    const char* e = std::getenv(name);
-    return e != nullptr && e[0] == '1' && e[1] == 0;
-}
-static bool prefill_stream_enabled()
-{
-    static const bool on = env_is_one("FLASHCK_PREFILL_STREAM");
-    return on;
-}
-static bool prefill_dma256_enabled()
-{
-    static const bool on = env_is_one("FLASHCK_PREFILL_DMA256");
-    return on;
-}
-
 static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t q_max_seq_len, bool uniform, void* stream,
-                          const char* what, int64_t max_keys_per_seq)
+                          const char* what)
 {
-    // the ping-pong kernel keeps one page id per key tile in LDS
-    const bool pp_uniform = uniform && max_keys_per_seq <= (int64_t)fck::kPrefillPageCache * fck::kPrefillKeyTile;
     if (q_max_seq_len <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_max_seq_len must be positive");
+    // The direct-to-LDS kernels address a tile's rows with 32-bit byte offsets from the tile's first row.
+    if ((int64_t)a.hk * d * 2 * 64 >= ((int64_t)1 << 31))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "kv_num_heads * head_dim = %ld is too large (64 cache rows must span < 2 GiB)", (long)(a.hk * d));
     // Long query runs at head dim <= 128 take the 8-wave ping-pong kernel (256 rows per workgroup); short runs and
     // head dim 256 take the 4-wave kernel (128 rows per workgroup).
     if (d <= 128 && q_max_seq_len > 128) {
         a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
-        const bool stream_uniform = uniform && max_keys_per_seq <= (int64_t)fck::kPrefillStreamRowCache * fck::kPrefillKeyTile;
-        if (prefill_stream_enabled() && stream_uniform && fck::prefill_stream_fits(a, cu_count()))
-            return launch_status(fck::launch_prefill_stream(a, (int)d, dtype, cu_count(), static_cast<hipStream_t>(stream)), what);
-        return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, pp_uniform, static_cast<hipStream_t>(stream)), what);
+        g_kernel = uniform ? "prefill_pp_kernel<uniform_page>" : "prefill_pp_kernel<row_lookup>";
+        return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }
     a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
-    if (d == 256 && pp_uniform && prefill_dma256_enabled())
-        return launch_status(fck::launch_prefill_dma(a, (int)d, dtype, static_cast<hipStream_t>(stream)), what);
+    g_kernel = uniform ? "prefill_kernel<uniform_page>" : "prefill_kernel<row_lookup>";
     return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
 }
 
@@ -321,6 +325,7 @@ int fck_fmha_fwd(const void* q, const void* k, const void* v, const void* bias, 
     a.window_left = window_left;
     a.window_right = window_right;
     a.kv.page_shift = -1;
+    a.kv.seqlen_k_ptr = seqlen_k_ptr;  // group mode: logical key counts of padded packed sequences
     if (seqstart_q) {
         a.kv.mode = 1;
         a.kv.seqstart_k = seqstart_k;
@@ -328,10 +333,9 @@ int fck_fmha_fwd(const void* q, const void* k, const void* v, const void* bias, 
         if (seqlen_q <= 0 || seqlen_k <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch mode needs seqlen_q, seqlen_k > 0");
         a.kv.mode = 0;
         a.kv.seqlen_k = (int32_t)seqlen_k;
-        a.kv.seqlen_k_ptr = seqlen_k_ptr;
         if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
     }
-    return prefill_common(a, d, dtype, q_max_seq_len, true, stream, "FmhaFwd launch", 0);
+    return prefill_common(a, d, dtype, q_max_seq_len, true, stream, "FmhaFwd launch");
 }
 
 int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
@@ -367,8 +371,9 @@ int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cac
     a.kv.kv_last_page_lens = kv_last_page_lens;
     a.kv.page_size = (int32_t)page_block_size;
     a.kv.page_shift = log2_exact(page_block_size);
-    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdBatchPrefill launch",
-                          num_total_pages * page_block_size);
+    if (num_total_pages * page_block_size > INT32_MAX)
+        return fail(FCK_ERR_INVALID_ARGUMENT, "a pool of %ld x %ld cache rows exceeds the 2^31 - 1 rows the kernels index", (long)num_total_pages, (long)page_block_size);
+    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdBatchPrefill launch");
 }
 
 int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
@@ -407,8 +412,7 @@ int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache
     a.kv.page_size = (int32_t)page_block_size;
     a.kv.page_shift = log2_exact(page_block_size);
     if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
-    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdPagedKV launch",
-                          batch_stride_block_table * page_block_size);
+    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdPagedKV launch");
 }
 
 }  // extern "C"

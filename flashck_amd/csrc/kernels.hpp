@@ -3,7 +3,30 @@
 
 #include "common.hpp"
 
+#include <mutex>
+
 namespace fck {
+
+// Launch `Kern` with `lds` bytes of dynamic LDS.  More than 64 KiB needs an opt-in per kernel and device; it is made
+// once per device under std::call_once, so concurrent first calls from several host threads are safe, and every later
+// call is a plain launch (nothing but the launch itself reaches the stream, so a warmed-up call can be captured).
+template <auto Kern, typename Args>
+inline hipError_t launch_with_lds(dim3 grid, dim3 block, size_t lds, hipStream_t st, const Args& a)
+{
+    constexpr int kMaxDev = 64;
+    static std::once_flag once[kMaxDev];
+    static hipError_t status[kMaxDev];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDev) return hipErrorInvalidDevice;
+    std::call_once(once[dev], [&] {
+        status[dev] = hipFuncSetAttribute((const void*)Kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
+    if (status[dev] != hipSuccess) return status[dev];
+    hipLaunchKernelGGL(Kern, grid, block, lds, st, a);
+    return hipGetLastError();
+}
 
 struct SplitKvArgs {
     const void* q;
@@ -14,6 +37,9 @@ struct SplitKvArgs {
     const int32_t* seqstart_q;
     KvAddr kv;
     int32_t batch, sq, hq, hk, num_splits;
+    int32_t m_tiles;     // row tiles per (sequence, KV head); set by the launcher
+    uint32_t* tickets;   // non-null: the last workgroup of a (sequence, head group, row tile) merges the splits into `o`
+    void* o;
     int64_t shape_sq;  // Sq of the workspace: sq (batch mode) or total_q (group mode)
     float scale_log2;  // scale * log2(e)
     uint32_t mask_type;
@@ -62,8 +88,10 @@ struct PrefillArgs {
     int64_t window_left, window_right;
 };
 
-hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page,
+hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page, int num_cu,
                                  hipStream_t st);
+// row tiles per (sequence, KV head) the split-KV launcher uses for `rows_max` packed query rows
+int splitkv_decode_m_tiles(int d, int rows_max);
 hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st);
 hipError_t launch_appendkv(const AppendKvArgs& a, int dtype, int max_new, hipStream_t st);
 hipError_t launch_prefill(const PrefillArgs& a, int d, int dtype, bool uniform_page, hipStream_t st);

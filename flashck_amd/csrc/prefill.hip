@@ -285,27 +285,8 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
 {
     const dim3 grid(a.m_tiles, a.hq, a.batch);
     constexpr size_t lds = prefill_lds_bytes<D>();
-    hipError_t e;
-    if (uniform) {
-        auto kern = prefill_kernel<T, D, true>;
-        static bool once = false;
-        if (!once) {
-            e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-            once = true;
-        }
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a);
-    } else {
-        auto kern = prefill_kernel<T, D, false>;
-        static bool once = false;
-        if (!once) {
-            e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-            once = true;
-        }
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a);
-    }
-    return hipGetLastError();
+    if (uniform) return launch_with_lds<prefill_kernel<T, D, true>>(grid, dim3(256), lds, st, a);
+    return launch_with_lds<prefill_kernel<T, D, false>>(grid, dim3(256), lds, st, a);
 }
 
 template <typename T>

@@ -334,15 +334,7 @@ static hipError_t launch_d(const PrefillArgs& a, hipStream_t st)
     const int g = a.hq / a.hk, gx = (a.batch * a.hk + 7) / 8;
     const dim3 grid(8 * a.m_tiles * gx * g);
     constexpr size_t lds = (size_t)4 * Shape<D>::TILEB + kPrefillPageCache * 4;
-    auto kern = prefill_dma_kernel<T, D>;
-    static bool once = false;
-    if (!once) {
-        const hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        once = true;
-    }
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a);
-    return hipGetLastError();
+    return launch_with_lds<prefill_dma_kernel<T, D>>(grid, dim3(256), lds, st, a);
 }
 
 }  // namespace dma

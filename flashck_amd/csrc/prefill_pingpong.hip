@@ -174,8 +174,8 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     }
 
     // First cache row of every tile (uniform-page path): computed once per workgroup into LDS, so the main loop needs
-    // one LDS read per tile and no table lookup.  The host only selects this path when a sequence cannot have more
-    // than kPrefillPageCache tiles.
+    // one LDS read per tile and no table lookup; tiles past the first kPrefillPageCache of a very long sequence are
+    // looked up one by one (tile_row0).
     constexpr int kPageCache = kPrefillPageCache;
     int FCK_LDS* row_lds = (int FCK_LDS*)(lds + 2 * kRing * S::TILEB);
     if constexpr (kUniformPage) {
@@ -191,6 +191,16 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     int row_vec = 0, row_chunk = -1;
     auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t {
         if (ks.table != nullptr) {
+            if (i >= kPageCache) {
+                // A sequence with more key tiles than the cache holds (> kPageCache * 64 keys): one table lookup per
+                // tile for the tiles past the cached ones.  A scalar load through the constant address space (the table
+                // is an input, never written here), consumed inside this branch so that the wait it needs stays here.
+                const int kb = (t_begin + i) * S::BN;
+                const int pi = a.kv.page_shift >= 0 ? kb >> a.kv.page_shift : kb / a.kv.page_size;
+                int page = ((const __attribute__((address_space(4))) int32_t*)ks.table)[pi];
+                asm volatile("" : "+s"(page));
+                return (int64_t)page * a.kv.page_size + (kb - pi * a.kv.page_size);
+            }
             if ((i >> 6) != row_chunk) {
                 row_chunk = i >> 6;
                 row_vec = row_lds[min(row_chunk * 64 + lane, kPageCache - 1)];
@@ -442,27 +452,8 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
     const int g = a.hq / a.hk, gx = (a.batch * a.hk + 7) / 8;
     const dim3 grid(8 * a.m_tiles * gx * g);
     constexpr size_t lds = (size_t)2 * PPShape<D, BN>::RING * PPShape<D, BN>::TILEB + kPrefillPageCache * 4;
-    hipError_t e;
-    if (uniform) {
-        auto kern = prefill_pp_kernel<T, D, BN, true>;
-        static bool once = false;
-        if (!once) {
-            e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-            once = true;
-        }
-        hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, a);
-    } else {
-        auto kern = prefill_pp_kernel<T, D, BN, false>;
-        static bool once = false;
-        if (!once) {
-            e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-            once = true;
-        }
-        hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, a);
-    }
-    return hipGetLastError();
+    if (uniform) return launch_with_lds<prefill_pp_kernel<T, D, BN, true>>(grid, dim3(512), lds, st, a);
+    return launch_with_lds<prefill_pp_kernel<T, D, BN, false>>(grid, dim3(512), lds, st, a);
 }
 
 // `a.m_tiles` must count 256-row tiles.  Key tile: 64 at head dim 64, 32 at head dim 128 (register budget of two

@@ -93,7 +93,7 @@ __device__ __forceinline__ KvSeq kv_seq_c(const KvAddr& a, int b)
         const int s0 = ldc(a.seqstart_k, b);
         s.table = nullptr;
         s.base_row = s0;
-        s.len = ldc(a.seqstart_k, b + 1) - s0;
+        s.len = a.seqlen_k_ptr ? ldc(a.seqlen_k_ptr, b) : ldc(a.seqstart_k, b + 1) - s0;
     } else if (a.mode == 2) {
         s.table = a.block_table + (int64_t)b * a.block_table_stride;
         s.base_row = 0;
@@ -603,15 +603,7 @@ static hipError_t launch_d(const PrefillArgs& a, int num_cu, hipStream_t st)
     const dim3 grid(8 * nwx);
     constexpr size_t lds = (size_t)2 * Shape<D>::RING * Shape<D>::TILEB + 2 * kPrefillStreamRowCache * 4 +
                            kPrefillStreamMaxItems * 4 + 64;
-    auto kern = prefill_stream_kernel<T, D>;
-    static bool once = false;
-    if (!once) {
-        const hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        once = true;
-    }
-    hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, a);
-    return hipGetLastError();
+    return launch_with_lds<prefill_stream_kernel<T, D>>(grid, dim3(512), lds, st, a);
 }
 
 }  // namespace stream

@@ -21,20 +21,7 @@ __global__ __launch_bounds__(256) void splitkv_combine_kernel(const CombineArgs 
     const int ns = a.num_splits;
     const int64_t w0 = ((b * a.hq + h) * ns) * a.Sq + i;  // split 0; next split is Sq further
 
-    float m = -INFINITY;
-    for (int s = 0; s < ns; ++s) m = fmaxf(m, a.lse_acc[w0 + s * a.Sq]);
-    float sum = 0.f;
-    if (m != -INFINITY)
-        for (int s = 0; s < ns; ++s) sum += __expf(a.lse_acc[w0 + s * a.Sq] - m);
-    const float L = (sum == 0.f) ? -INFINITY : __logf(sum) + m;
-
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    if (L != -INFINITY)
-        for (int s = 0; s < ns; ++s) {
-            const float w = __expf(a.lse_acc[w0 + s * a.Sq] - L);
-            const f32x4_t v = *reinterpret_cast<const f32x4_t*>(a.o_acc + (w0 + s * a.Sq) * DV + c);
-            acc += w * v;
-        }
+    const f32x4_t acc = combine_splits<DV>(a.lse_acc, a.o_acc, w0, a.Sq, ns, c);
     u32x2_t out;
     out[0] = T::pack2(acc[0], acc[1]);
     out[1] = T::pack2(acc[2], acc[3]);

@@ -34,6 +34,10 @@ ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALF_ROTATED = 0, 1, 2
 _DTYPE_ID = {torch.float16: 3, torch.bfloat16: 4}  # flashck::DataType, core/utils/dtype.h:16-28
 
 
+# Host-side tests of the validation code switch this off (and replace _call); nothing else may.
+_REQUIRE_GPU_TENSORS = True
+
+
 def _dtype_id(t: torch.Tensor) -> int:
     if t.dtype not in _DTYPE_ID:
         raise TypeError(f"FMHA supports torch.float16 and torch.bfloat16, got {t.dtype}")
@@ -47,7 +51,7 @@ def _check_tensor(name, t, dtype=None, ndim=None, optional=False):
         raise TypeError(f"{name} must be a torch.Tensor, got None")
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"Expected {name} to be a torch.Tensor, got {type(t)}")
-    if not t.is_cuda:
+    if _REQUIRE_GPU_TENSORS and not t.is_cuda:
         raise ValueError(f"{name} must live on the GPU (got device {t.device})")
     if not t.is_contiguous():
         raise ValueError(f"{name} must be contiguous")
@@ -55,6 +59,36 @@ def _check_tensor(name, t, dtype=None, ndim=None, optional=False):
         raise TypeError(f"{name} must have dtype {dtype}, got {t.dtype}")
     if ndim is not None and t.dim() not in (ndim if isinstance(ndim, tuple) else (ndim,)):
         raise ValueError(f"{name} must have {ndim} dimensions, got shape {tuple(t.shape)}")
+
+
+def _check_shape(name, t, shape, like):
+    """A caller-supplied buffer (workspace or output) must be exactly what the kernel is about to write: the C ABI
+    only sees a pointer, so a wrong size here would be an out-of-bounds write on the GPU."""
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    if t.device != like.device:
+        raise ValueError(f"{name} is on {t.device}, the inputs are on {like.device}")
+
+
+def _out(name, out, shape, dtype, like):
+    """`out` validated against (shape, dtype, device of `like`), or a new tensor when it is None."""
+    if out is None:
+        return torch.empty(*shape, dtype=dtype, device=like.device)
+    _check_tensor(name, out, dtype=dtype)
+    _check_shape(name, out, shape, like)
+    return out
+
+
+def _check_kv(q, k, v, ndim):
+    """k and v against q: same rank, k's head dim is q's, v agrees with k on everything but the head dim."""
+    if k.dim() != ndim or v.dim() != ndim:
+        raise ValueError(f"k {tuple(k.shape)} / v {tuple(v.shape)} must have {ndim} dimensions")
+    if k.shape[-1] != q.shape[-1]:
+        raise ValueError(f"k head dim {k.shape[-1]} != q head dim {q.shape[-1]}")
+    if v.shape[:-1] != k.shape[:-1]:
+        raise ValueError(f"v {tuple(v.shape)} does not match k {tuple(k.shape)}")
+    if k.shape[-2] <= 0 or q.shape[-2] % k.shape[-2]:
+        raise ValueError(f"q heads {q.shape[-2]} must be a multiple of kv heads {k.shape[-2]}")
 
 
 def _ptr(t):
@@ -108,12 +142,15 @@ def fmha_fwd(q, k, v, scale: float = 0.0, mask_type: int = MASK_NONE, window: Tu
     _check_tensor("v", v, dtype=q.dtype, ndim=4)
     _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1, optional=True)
     B, sq, Hq, D = q.shape
-    if k.shape[0] != B or v.shape[:3] != k.shape[:3]:
+    _check_kv(q, k, v, 4)
+    if k.shape[0] != B:
         raise ValueError(f"k {tuple(k.shape)} / v {tuple(v.shape)} do not match q {tuple(q.shape)}")
     if q.numel() == 0:
         raise ValueError("Input tensor cannot be empty")
+    if seqlen_k is not None and seqlen_k.numel() != B:
+        raise ValueError(f"seqlen_k must have {B} entries, got {seqlen_k.numel()}")
     sk, Hk, Dv = k.shape[1], k.shape[2], v.shape[3]
-    o = out if out is not None else torch.empty(B, sq, Hq, Dv, dtype=q.dtype, device=q.device)
+    o = _out("out", out, (B, sq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
     _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), None, None, _ptr(seqlen_k), B, sq, sk, Hq, Hk, D, Dv,
           sq, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
@@ -121,8 +158,10 @@ def fmha_fwd(q, k, v, scale: float = 0.0, mask_type: int = MASK_NONE, window: Tu
 
 
 def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scale: float = 0.0,
-                    mask_type: int = MASK_NONE, window=(-1, -1), out=None) -> torch.Tensor:
-    """Dense attention, group mode: q [total_q,Hq,D], k/v [total_k,Hk,D] packed by cu_seqlens."""
+                    mask_type: int = MASK_NONE, window=(-1, -1), seqlen_k=None, out=None) -> torch.Tensor:
+    """Dense attention, group mode: q [total_q,Hq,D], k/v [total_k,Hk,D] packed by cu_seqlens.
+
+    seqlen_k (int32 [B], optional): logical key counts when the packed K/V slots hold padding behind the keys."""
     _check_tensor("q", q, ndim=3)
     _check_tensor("k", k, dtype=q.dtype, ndim=3)
     _check_tensor("v", v, dtype=q.dtype, ndim=3)
@@ -132,10 +171,14 @@ def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scal
         raise ValueError("cu_seqlens_q and cu_seqlens_k must both have batch + 1 entries")
     B = cu_seqlens_q.numel() - 1
     tq, Hq, D = q.shape
+    _check_kv(q, k, v, 3)
+    _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1, optional=True)
+    if seqlen_k is not None and seqlen_k.numel() != B:
+        raise ValueError(f"seqlen_k must have {B} entries, got {seqlen_k.numel()}")
     Hk, Dv = k.shape[1], v.shape[2]
-    o = out if out is not None else torch.empty(tq, Hq, Dv, dtype=q.dtype, device=q.device)
+    o = _out("out", out, (tq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
-    _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), None, B, tq,
+    _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), _ptr(seqlen_k), B, tq,
           k.shape[0], Hq, Hk, D, Dv, max_seqlen_q, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
     return o
 
@@ -157,6 +200,7 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
     if int(num_splits) < 1:
         raise ValueError("num_splits must be >= 1")
     Hq, D = q.shape[-2], q.shape[-1]
+    _check_kv(q, k, v, 3 if (cu_seqlens_k is not None and block_table is None) else 4)
     Hk, Dv = k.shape[-2], v.shape[-1]
     if group:
         B, sq, bs = cu_seqlens_q.numel() - 1, q.shape[0], 1
@@ -165,6 +209,8 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
     else:
         B, sq, bs = q.shape[0], q.shape[1], q.shape[0]
         max_seqlen_q = sq
+    if seqlen_k is not None and seqlen_k.numel() != B:
+        raise ValueError(f"seqlen_k must have {B} entries, got {seqlen_k.numel()}")
     if block_table is not None:
         if seqlen_k is None:
             raise ValueError("a paged cache needs seqlen_k")
@@ -174,8 +220,16 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
     else:
         page, max_blocks = 0, 0
         sk = k.shape[0] if cu_seqlens_k is not None else k.shape[1]
-    if o_acc is None or lse_acc is None:
+    if (o_acc is None) != (lse_acc is None):
+        raise ValueError("o_acc and lse_acc must be given together")
+    if o_acc is None:
         o_acc, lse_acc = splitkv_workspace(bs, Hq, sq, Dv, num_splits, q.device)
+    else:
+        # the kernel writes with the strides of THIS split count
+        _check_tensor("o_acc", o_acc, dtype=torch.float32)
+        _check_tensor("lse_acc", lse_acc, dtype=torch.float32)
+        _check_shape("o_acc", o_acc, (bs, Hq, int(num_splits), sq, Dv), q)
+        _check_shape("lse_acc", lse_acc, (bs, Hq, int(num_splits), sq), q)
     wl, wr = _window(window)
     _call("fck_fmha_fwd_splitkv", _ptr(q), _ptr(k), _ptr(v), None, _ptr(lse_acc), _ptr(o_acc), _ptr(cu_seqlens_q),
           _ptr(cu_seqlens_k), _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv,
@@ -193,12 +247,16 @@ def fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype, cu_seqlens_q=None, max_seqle
     bs, Hq, ns, sq, Dv = o_acc.shape
     if tuple(lse_acc.shape) != (bs, Hq, ns, sq):
         raise ValueError(f"lse_acc {tuple(lse_acc.shape)} does not match o_acc {tuple(o_acc.shape)}")
+    if lse_acc.device != o_acc.device:
+        raise ValueError(f"lse_acc is on {lse_acc.device}, o_acc on {o_acc.device}")
     if cu_seqlens_q is not None:
+        if bs != 1:
+            raise ValueError(f"group mode partials have shape batch 1, got {bs}")
         B = cu_seqlens_q.numel() - 1
-        o = out if out is not None else torch.empty(sq, Hq, Dv, dtype=dtype, device=o_acc.device)
+        o = _out("out", out, (sq, Hq, Dv), dtype, o_acc)
     else:
         B = bs
-        o = out if out is not None else torch.empty(bs, sq, Hq, Dv, dtype=dtype, device=o_acc.device)
+        o = _out("out", out, (bs, sq, Hq, Dv), dtype, o_acc)
     _call("fck_fmha_fwd_splitkv_combine", _ptr(lse_acc), _ptr(o_acc), _ptr(o), _ptr(cu_seqlens_q), B, sq, Hq, Dv,
           max_seqlen_q or sq, ns, _DTYPE_ID[dtype], _stream())
     return o
@@ -226,6 +284,21 @@ def fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, *, cu_seqlens_k
     B = seqlen_k.numel()
     Hk, D, Dv = knew.shape[-2], knew.shape[-1], vnew.shape[-1]
     Hq = q.shape[-2] if q is not None else 0
+    if k_cache.shape[2:] != (Hk, D) or v_cache.shape[2:] != (Hk, Dv) or v_cache.shape[:2] != k_cache.shape[:2]:
+        raise ValueError(f"k_cache {tuple(k_cache.shape)} / v_cache {tuple(v_cache.shape)} do not match knew "
+                         f"{tuple(knew.shape)} / vnew {tuple(vnew.shape)}")
+    if vnew.shape[:-1] != knew.shape[:-1]:
+        raise ValueError(f"vnew {tuple(vnew.shape)} does not match knew {tuple(knew.shape)}")
+    if q is not None and (q.shape[-1] != D or q.shape[:-2] != knew.shape[:-2] or Hq % Hk):
+        raise ValueError(f"q {tuple(q.shape)} does not match knew {tuple(knew.shape)}")
+    if packed and cu_seqlens_knew.numel() != B + 1:
+        raise ValueError(f"cu_seqlens_knew must have {B + 1} entries, got {cu_seqlens_knew.numel()}")
+    if not packed and knew.shape[0] != B:
+        raise ValueError(f"knew batch {knew.shape[0]} != number of sequences {B}")
+    if block_table is not None and (block_table.dim() != 2 or block_table.shape[0] != B):
+        raise ValueError(f"block_table must be [batch, max_pages_per_seq] with batch {B}, got {tuple(block_table.shape)}")
+    if rope_mode != ROPE_NONE and rotary_cos is not None and rotary_sin is not None and rotary_cos.shape != rotary_sin.shape:
+        raise ValueError("rotary_cos and rotary_sin must have the same shape")
     if packed:
         if max_seqlen_knew <= 0:
             raise ValueError("packed new tokens need max_seqlen_knew")
@@ -262,8 +335,11 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
     if kv_indptr.numel() != B + 1:
         raise ValueError("kv_indptr must have batch + 1 entries")
     tq, Hq, D = q.shape
+    _check_kv(q, k_cache, v_cache, 4)
+    if kv_last_page_lens is not None and kv_last_page_lens.numel() != B:
+        raise ValueError(f"kv_last_page_lens must have {B} entries, got {kv_last_page_lens.numel()}")
     num_pages, page, Hk, Dv = v_cache.shape
-    o = out if out is not None else torch.empty(tq, Hq, Dv, dtype=q.dtype, device=q.device)
+    o = _out("out", out, (tq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
     _call("fck_fmha_batch_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
           _ptr(kv_page_indices), _ptr(kv_last_page_lens), num_pages, page, B, Hq, Hk, D, Dv, max_seqlen_q,
@@ -283,11 +359,16 @@ def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q
     _check_tensor("cu_seqlens_q", cu_seqlens_q, dtype=torch.int32, ndim=1, optional=True)
     B = seqlen_k.numel()
     Hq, D = q.shape[-2], q.shape[-1]
+    _check_kv(q, k_cache, v_cache, 4)
+    if block_table.shape[0] != B:
+        raise ValueError(f"block_table must be [batch, max_pages_per_seq] with batch {B}, got {tuple(block_table.shape)}")
+    if (cu_seqlens_q.numel() - 1 if group else q.shape[0]) != B:
+        raise ValueError("seqlen_k must have one entry per sequence of q")
     _, page, Hk, Dv = v_cache.shape
     sq = 0 if group else q.shape[1]
     if group and max_seqlen_q <= 0:
         raise ValueError("group mode needs max_seqlen_q")
-    o = out if out is not None else torch.empty(*q.shape[:-1], Dv, dtype=q.dtype, device=q.device)
+    o = _out("out", out, (*q.shape[:-1], Dv), q.dtype, q)
     wl, wr = _window(window)
     _call("fck_fmha_fwd_pagedkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
           _ptr(block_table), block_table.shape[1], page, B, sq, Hq, Hk, D, Dv, max_seqlen_q or sq, _scale(scale, D), wl, wr,
@@ -308,10 +389,20 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
                       window=(-1, -1), workspace=None, out=None) -> torch.Tensor:
     """Paged decode = split-KV forward + LSE combine; num_splits = 0 asks the heuristic (needs max_seqlen_k)."""
     group = cu_seqlens_q is not None
+    _check_tensor("q", q, ndim=3 if group else 4)
+    _check_tensor("k_cache", k_cache, dtype=q.dtype, ndim=4)
+    _check_tensor("v_cache", v_cache, dtype=q.dtype, ndim=4)
+    _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1)
+    _check_tensor("block_table", block_table, dtype=torch.int32, ndim=2)
     Hq, D = q.shape[-2], q.shape[-1]
     Hk = k_cache.shape[2]
     B = seqlen_k.numel()
     sq = max_seqlen_q if group else q.shape[1]
+    if workspace is not None and num_splits <= 0:
+        # the partials are laid out for one split count: with a caller-owned workspace that count is the workspace's
+        num_splits = int(workspace[0].shape[2]) if workspace[0].dim() == 5 else 0
+        if num_splits <= 0:
+            raise ValueError("workspace must be (o_acc [Bs,Hq,ns,Sq,Dv], lse_acc [Bs,Hq,ns,Sq])")
     if num_splits <= 0:
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * k_cache.shape[1]

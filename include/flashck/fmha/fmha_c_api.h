@@ -62,6 +62,11 @@ FCK_EXPORT const char* fck_last_error(void);
 /* Library version string. */
 FCK_EXPORT const char* fck_fmha_version(void);
 
+/* Name of the kernel family (and addressing variant) the calling thread's last successful dispatch chose, "" before
+ * the first one.  For tests and tuning records; FlashCK logs the same through its instance names
+ * (core/profiling/attention/fmha_fwd_split_kv/fmha_fwd_split_kv_codegen.cc:60-94). */
+FCK_EXPORT const char* fck_fmha_last_kernel(void);
+
 /*
  * Dense / varlen forward.  Replaces `FmhaFwd`, fmha_fwd/fmha_fwd_jinja.h:124-147 (args :68-122, strides :186-304).
  * batch mode: seqstart_q = seqstart_k = NULL; seqlen_k_ptr optional per-batch key counts.

@@ -168,7 +168,9 @@ static int seq_k_len(const fck_orc_problem* p, int b)
 {
     switch (p->kv_mode) {
     case FCK_ORC_KV_BATCH: return p->seqlen_k ? p->seqlen_k[b] : p->sk;
-    case FCK_ORC_KV_GROUP: return p->seqstart_k[b + 1] - p->seqstart_k[b];
+    /* ck_tile/ops/fmha/kernel/fmha_fwd_splitkv_kernel.hpp:648-650: seqlen_k_ptr, when given, is the logical length of
+       a packed sequence whose slot [seqstart_k[b], seqstart_k[b+1]) may hold padding behind it */
+    case FCK_ORC_KV_GROUP: return p->seqlen_k ? p->seqlen_k[b] : p->seqstart_k[b + 1] - p->seqstart_k[b];
     case FCK_ORC_KV_BLOCK_TABLE: return p->seqlen_k[b];
     case FCK_ORC_KV_PAGE_LIST: {
         int np = p->kv_indptr[b + 1] - p->kv_indptr[b];

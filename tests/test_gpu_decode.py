@@ -62,6 +62,23 @@ def test_paged_multi_query_causal(fmha, orc, sq, hq, hk):
     _run_paged(fmha, orc, kv, 2, mask_type=2, window=(17, 0))      # sliding window
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d,page", [(128, 128), (64, 64), (128, 48)])
+def test_paged_decode_head_pairs(fmha, orc, dtype, d, page):
+    """Grids of at least one workgroup per CU take the kernel that streams two KV heads per workgroup (16-key tiles):
+    20 sequences x 8 KV heads x 4 splits.  Lengths around the 16-key tile and page borders; page 48 is not a multiple
+    of the tile, so it takes the per-row lookup variant."""
+    g = torch.Generator().manual_seed(31 + d + page)
+    lens = [1, 15, 16, 17, 47, 48, 49, 95, 96, 97, 127, 128, 129, 255, 256, 257, 700, 1023, 1500, 33]
+    kv = gen.paged_kv(lens, 8, d, dtype, g, page)
+    kv["q"] = gen.randn((len(lens), 1, 32, d), dtype, g)
+    kv["scale"] = 1 / math.sqrt(d)
+    _run_paged(fmha, orc, kv, 4)
+    from flashck_amd import _lib
+    assert b"splitkv_decode_kernel" in _lib.load().fck_fmha_last_kernel()
+    _run_paged(fmha, orc, kv, 4, mask_type=2, window=(40, 0))  # sliding window: leading tiles are skipped
+
+
 def test_group_mode_ragged_queries(fmha, orc):
     # ragged query counts (1..16 new tokens per sequence) through seqstart_q
     g = torch.Generator().manual_seed(5)

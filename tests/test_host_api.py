@@ -105,3 +105,71 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libflashck_fmha.so"))
     with pytest.raises(_lib.FlashCKLibraryError):
         _lib.load()
+
+
+@pytest.fixture()
+def host_ops(monkeypatch):
+    """The Python operators with the GPU-residency check off and the C call recorded instead of made, so that the
+    shape / dtype validation in front of the C ABI can be exercised with CPU tensors."""
+    calls = []
+    monkeypatch.setattr(fmha.fmha, "_REQUIRE_GPU_TENSORS", False)
+    monkeypatch.setattr(fmha.fmha, "_call", lambda name, *a: calls.append(name))
+    monkeypatch.setattr(fmha.fmha, "_stream", lambda: None)
+    return calls
+
+
+def test_caller_supplied_buffers_are_validated(host_ops):
+    T = torch.bfloat16
+    B, Hq, Hk, D, P, ns = 2, 4, 2, 64, 16, 3
+    q = torch.zeros(B, 1, Hq, D, dtype=T)
+    kc, vc = torch.zeros(8, P, Hk, D, dtype=T), torch.zeros(8, P, Hk, D, dtype=T)
+    sl = torch.full((B,), 20, dtype=torch.int32)
+    bt = torch.zeros(B, 4, dtype=torch.int32)
+    o_acc, lse_acc = torch.zeros(B, Hq, ns, 1, D), torch.zeros(B, Hq, ns, 1)
+    fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, o_acc=o_acc, lse_acc=lse_acc)
+    assert host_ops == ["fck_fmha_fwd_splitkv"]
+    # a workspace laid out for another split count would be written out of bounds
+    with pytest.raises(ValueError, match="o_acc must have shape"):
+        fmha.fmha_fwd_splitkv(q, kc, vc, ns + 1, seqlen_k=sl, block_table=bt, o_acc=o_acc, lse_acc=lse_acc)
+    with pytest.raises(ValueError, match="lse_acc must have shape"):
+        fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, o_acc=o_acc, lse_acc=lse_acc[:, :, :2].contiguous())
+    with pytest.raises(TypeError, match="o_acc"):
+        fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, o_acc=o_acc.half(), lse_acc=lse_acc)
+    with pytest.raises(ValueError, match="together"):
+        fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, o_acc=o_acc)
+    # k with another head dim, v that disagrees with k, wrong rank
+    with pytest.raises(ValueError, match="head dim"):
+        fmha.fmha_fwd_splitkv(q, torch.zeros(8, P, Hk, 128, dtype=T), vc, ns, seqlen_k=sl, block_table=bt)
+    with pytest.raises(ValueError, match="does not match k"):
+        fmha.fmha_fwd_splitkv(q, kc, torch.zeros(8, P, 1, D, dtype=T), ns, seqlen_k=sl, block_table=bt)
+    with pytest.raises(ValueError, match="dimensions"):
+        fmha.fmha_fwd_splitkv(q, kc[0], vc[0], ns, seqlen_k=sl, block_table=bt)
+    # decode with a caller-owned workspace and num_splits = 0: the workspace's split count is the one used
+    del host_ops[:]
+    fmha.fmha_decode_paged(q, kc, vc, sl, bt, num_splits=0, workspace=(o_acc, lse_acc))
+    assert host_ops == ["fck_fmha_fwd_splitkv", "fck_fmha_fwd_splitkv_combine"]
+    with pytest.raises(ValueError, match="o_acc must have shape"):
+        fmha.fmha_decode_paged(q, kc, vc, sl, bt, num_splits=5, workspace=(o_acc, lse_acc))
+    # out= of every operator
+    with pytest.raises(ValueError, match="out must have shape"):
+        fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, T, out=torch.zeros(B, 1, Hq, D - 8, dtype=T))
+    with pytest.raises(TypeError, match="out"):
+        fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, T, out=torch.zeros(B, 1, Hq, D, dtype=torch.float16))
+    qd = torch.zeros(B, 5, Hq, D, dtype=T)
+    kd = torch.zeros(B, 7, Hk, D, dtype=T)
+    with pytest.raises(ValueError, match="out must have shape"):
+        fmha.fmha_fwd(qd, kd, kd, out=torch.zeros(B, 4, Hq, D, dtype=T))
+    with pytest.raises(ValueError, match="out must have shape"):
+        fmha.fmha_fwd_pagedkv(qd, kc, vc, sl, bt, out=torch.zeros(B, 5, Hq, 2 * D, dtype=T))
+    cu = torch.tensor([0, 3, 5], dtype=torch.int32)
+    qp = torch.zeros(5, Hq, D, dtype=T)
+    with pytest.raises(ValueError, match="out must have shape"):
+        fmha.fmha_batch_prefill(qp, kc, vc, cu, torch.tensor([0, 1, 2], dtype=torch.int32),
+                                torch.tensor([0, 1], dtype=torch.int32), max_seqlen_q=3, out=torch.zeros(4, Hq, D, dtype=T))
+    with pytest.raises(ValueError, match="out must have shape"):
+        fmha.fmha_fwd_varlen(qp, torch.zeros(9, Hk, D, dtype=T), torch.zeros(9, Hk, D, dtype=T), cu, cu, 3,
+                             out=torch.zeros(5, Hq, D + 8, dtype=T))
+    # appendkv: caches that do not match the new tokens
+    kn = torch.zeros(B, 1, Hk, D, dtype=T)
+    with pytest.raises(ValueError, match="do not match knew"):
+        fmha.fmha_fwd_appendkv(None, kc, torch.zeros(8, P, Hk, 32, dtype=T), kn, kn, sl, block_table=bt)
