@@ -118,7 +118,7 @@ def bench_decode(args, torch, fmha, gen, which):
         if ev is not None:
             ev[0].record()
         if fused:
-            raise SystemExit("this build has no fused decode entry point")
+            fmha.fmha_fwd_splitkv_fused(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], out=o)
         else:
             fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc)
         if ev is not None:

@@ -19,6 +19,7 @@ SIGNATURES = {
     "fck_fmha_last_kernel": (ctypes.c_char_p, []),
     "fck_fmha_fwd": (ctypes.c_int, [_vp] * 8 + [_i64] * 8 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_fwd_splitkv": (ctypes.c_int, [_vp] * 11 + [_i64] * 11 + [_f32, _i64, _i64, _u32, _i32, _vp]),
+    "fck_fmha_fwd_splitkv_fused": (ctypes.c_int, [_vp] * 10 + [_i64] * 11 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_fwd_splitkv_combine": (ctypes.c_int, [_vp] * 4 + [_i64] * 6 + [_i32, _vp]),
     "fck_fmha_fwd_appendkv": (ctypes.c_int, [_vp] * 7 + [_i64, _vp, _vp, _i64, _i32, _i32, _vp, _i64, _i64, _vp]
                               + [_i64] * 6 + [_i32, _vp]),

@@ -200,6 +200,52 @@ int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v, const void
                          "FmhaFwdSplitKV launch");
 }
 
+int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, const void* bias, void* o,
+                               const int32_t* seqstart_q, const int32_t* seqstart_k, const int32_t* seqlen_k_ptr,
+                               const int32_t* block_table, const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
+                               int64_t seqlen_k, int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len,
+                               int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size, float scale,
+                               int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream)
+{
+    g_err[0] = 0;
+    // num_splits == 0: the split count comes from the CU count and the longest possible KV length (the capacity of
+    // the block table, or seqlen_k), as fck_fmha_num_splits_heuristic gives it
+    if (num_splits == 0) {
+        const int64_t max_sk = block_table ? (batch > 0 ? max_num_page_blocks / batch : 0) * page_block_size : seqlen_k;
+        if (max_sk <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "num_splits = 0 needs a positive key-count bound (seqlen_k or the block table's capacity)");
+        num_splits = fck_fmha_num_splits_heuristic(batch, hq, hk, q_max_seq_len > 0 ? q_max_seq_len : seqlen_q, max_sk, d, 0);
+    }
+    fck::SplitKvArgs a;
+    bool uniform;
+    int rows_max;
+    if (int rc = splitkv_setup(a, uniform, rows_max, q, k, v, bias, seqstart_q, seqstart_k, seqlen_k_ptr, block_table,
+                               cache_batch_idx, batch, seqlen_q, seqlen_k, hq, hk, d, dv, q_max_seq_len, num_splits,
+                               max_num_page_blocks, page_block_size, scale, window_left, window_right, mask_type, dtype))
+        return rc;
+    if (!o) return fail(FCK_ERR_INVALID_ARGUMENT, "o must not be null");
+    if (!aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "o must be 16-byte aligned");
+    // The partial results and the arrival tickets live in a fixed device array of the library: nothing is allocated.
+    const int64_t shape_batch = seqstart_q ? 1 : batch;
+    const int64_t part_rows = shape_batch * hq * num_splits * seqlen_q;
+    const int64_t m_tiles = fck::splitkv_decode_m_tiles((int)d, rows_max);
+    const int64_t tickets = batch * hk * m_tiles;
+    if (part_rows * (dv + 1) > fck::kDecodeScratchPartialFloats || tickets > fck::kDecodeScratchTickets)
+        return fail(FCK_ERR_UNSUPPORTED,
+                    "the fused split-KV entry point holds at most %ld partial floats (asked: %ld = rows %ld x (Dv + 1)) and %ld "
+                    "tickets (asked: %ld); use fck_fmha_fwd_splitkv + fck_fmha_fwd_splitkv_combine with a caller-owned workspace",
+                    (long)fck::kDecodeScratchPartialFloats, (long)(part_rows * (dv + 1)), (long)part_rows,
+                    (long)fck::kDecodeScratchTickets, (long)tickets);
+    float* scratch = nullptr;
+    if (hipError_t e = fck::decode_scratch(&scratch); e != hipSuccess) return launch_status(e, "scratch symbol lookup");
+    a.tickets = reinterpret_cast<uint32_t*>(scratch);
+    a.o_acc = scratch + fck::kDecodeScratchTickets;
+    a.lse_acc = a.o_acc + part_rows * dv;
+    a.o = o;
+    g_kernel = uniform ? "splitkv_decode_kernel<uniform_page,fused>" : "splitkv_decode_kernel<row_lookup,fused>";
+    return launch_status(fck::launch_splitkv_decode(a, (int)d, dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
+                         "FmhaFwdSplitKV (fused) launch");
+}
+
 int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o, const int32_t* seqstart_q, int64_t batch,
                                  int64_t seqlen_q, int64_t hq, int64_t dv, int64_t q_max_seq_len, int64_t num_splits,
                                  int32_t dtype, void* stream)

@@ -90,6 +90,12 @@ struct PrefillArgs {
 
 hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page, int num_cu,
                                  hipStream_t st);
+// Device memory the fused split-KV entry point uses instead of a caller-owned workspace: a fixed array in the library
+// (one copy per GPU): kDecodeScratchTickets arrival counters (self-resetting), then the partial results.
+constexpr int64_t kDecodeScratchTickets = 16384;
+constexpr int64_t kDecodeScratchPartialFloats = (int64_t)4 << 20;  // 16 MiB
+// address of the array on the current device (looked up once per device)
+hipError_t decode_scratch(float** ptr);
 // row tiles per (sequence, KV head) the split-KV launcher uses for `rows_max` packed query rows
 int splitkv_decode_m_tiles(int d, int rows_max);
 hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st);

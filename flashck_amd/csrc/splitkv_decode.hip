@@ -482,6 +482,29 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
 }
 
 // ------------------------------------------------------------------------------------------------------
+// Workspace of the fused entry point.  In host code the array's name is only a handle: its device address is looked up
+// per device with hipGetSymbolAddress, and only that address is ever handed to a kernel.
+static __device__ __align__(256) float g_decode_scratch[kDecodeScratchTickets + kDecodeScratchPartialFloats];
+
+hipError_t decode_scratch(float** ptr)
+{
+    constexpr int kMaxDev = 64;
+    static std::once_flag once[kMaxDev];
+    static hipError_t status[kMaxDev];
+    static float* addr[kMaxDev];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDev) return hipErrorInvalidDevice;
+    std::call_once(once[dev], [&] {
+        void* p = nullptr;
+        status[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(g_decode_scratch));
+        addr[dev] = static_cast<float*>(p);
+    });
+    *ptr = addr[dev];
+    return status[dev];
+}
+
 template <typename T, int D, int NW, int MB, int HG>
 static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
 {

@@ -23,6 +23,7 @@ from ...utils import FlashCKOperationType, register_flashck_functions, tuning
 __all__ = [
     "MASK_NONE", "MASK_TOP_LEFT", "MASK_BOTTOM_RIGHT", "MASK_GENERIC", "ROPE_NONE", "ROPE_INTERLEAVED",
     "ROPE_HALF_ROTATED", "fmha_fwd", "fmha_fwd_varlen", "fmha_fwd_splitkv", "fmha_fwd_splitkv_combine",
+    "fmha_fwd_splitkv_fused", "fused_splitkv_fits",
     "fmha_fwd_appendkv", "fmha_batch_prefill", "fmha_fwd_pagedkv", "fmha_decode_paged", "fmha_decode_step",
     "tune_decode_num_splits", "DecodeWorkspace", "num_splits_heuristic", "splitkv_workspace",
 ]
@@ -237,6 +238,69 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
     return o_acc, lse_acc
 
 
+# limits of the fused entry point's fixed device array (fmha_c_api.h, fck_fmha_fwd_splitkv_fused)
+_FUSED_MAX_PARTIAL_FLOATS = 4 << 20
+_FUSED_MAX_TICKETS = 16384
+_FUSED_MAX_AUTO_SPLITS = 128
+
+
+def fused_splitkv_fits(shape_batch, batch, q_num_heads, kv_num_heads, shape_seqlen_q, max_seqlen_q, v_head_dim, num_splits) -> bool:
+    """Whether fmha_fwd_splitkv_fused can hold this problem's partial results (num_splits = 0: worst case of the
+    library's own choice)."""
+    ns = num_splits if num_splits > 0 else _FUSED_MAX_AUTO_SPLITS
+    rows = max_seqlen_q * (q_num_heads // max(kv_num_heads, 1))
+    m_tiles = 1 if rows <= 32 else (rows + 31) // 32
+    return (shape_batch * q_num_heads * ns * shape_seqlen_q * (v_head_dim + 1) <= _FUSED_MAX_PARTIAL_FLOATS
+            and batch * kv_num_heads * m_tiles <= _FUSED_MAX_TICKETS)
+
+
+def fmha_fwd_splitkv_fused(q, k, v, num_splits: int = 0, *, seqlen_k=None, block_table=None, cache_batch_idx=None,
+                           cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q: int = 0, scale: float = 0.0,
+                           mask_type: int = MASK_NONE, window=(-1, -1), out=None) -> torch.Tensor:
+    """Split-KV forward + LSE combine in one launch that allocates nothing on the GPU side: the partial results live in
+    a fixed device array of the library (limits: see fused_splitkv_fits; beyond them NotImplementedError).
+
+    num_splits = 0 lets the library take its heuristic split count for the CU count and the longest possible KV length.  Calls that overlap in time on one GPU (different streams) race on that array; calls on one stream are safe.
+    Arguments as fmha_fwd_splitkv; returns o [B,sq,Hq,Dv] (or [total_q,Hq,Dv] in group mode).
+    """
+    group = cu_seqlens_q is not None
+    _check_tensor("q", q, ndim=3 if group else 4)
+    _check_tensor("k", k, dtype=q.dtype)
+    _check_tensor("v", v, dtype=q.dtype)
+    for name, t in (("seqlen_k", seqlen_k), ("block_table", block_table), ("cache_batch_idx", cache_batch_idx),
+                    ("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
+        _check_tensor(name, t, dtype=torch.int32, optional=True)
+    if int(num_splits) < 0:
+        raise ValueError("num_splits must be >= 0")
+    Hq, D = q.shape[-2], q.shape[-1]
+    _check_kv(q, k, v, 3 if (cu_seqlens_k is not None and block_table is None) else 4)
+    Hk, Dv = k.shape[-2], v.shape[-1]
+    if group:
+        B, sq = cu_seqlens_q.numel() - 1, q.shape[0]
+        if max_seqlen_q <= 0:
+            raise ValueError("group mode needs max_seqlen_q")
+    else:
+        B, sq = q.shape[0], q.shape[1]
+        max_seqlen_q = sq
+    if seqlen_k is not None and seqlen_k.numel() != B:
+        raise ValueError(f"seqlen_k must have {B} entries, got {seqlen_k.numel()}")
+    if block_table is not None:
+        if seqlen_k is None:
+            raise ValueError("a paged cache needs seqlen_k")
+        if block_table.dim() != 2 or block_table.shape[0] != B:
+            raise ValueError(f"block_table must be [batch, max_pages_per_seq], got {tuple(block_table.shape)}")
+        page, sk, max_blocks = k.shape[1], 0, block_table.numel()
+    else:
+        page, max_blocks = 0, 0
+        sk = k.shape[0] if cu_seqlens_k is not None else k.shape[1]
+    o = _out("out", out, (*q.shape[:-1], Dv), q.dtype, q)
+    wl, wr = _window(window)
+    _call("fck_fmha_fwd_splitkv_fused", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k),
+          _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv, max_seqlen_q, int(num_splits),
+          max_blocks, page, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    return o
+
+
 def fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype, cu_seqlens_q=None, max_seqlen_q: int = 0, out=None) -> torch.Tensor:
     """LSE combine of split-KV partials -> o [B,sq,Hq,Dv] (or [total_q,Hq,Dv] in group mode)."""
     if dtype not in _DTYPE_ID:
@@ -386,8 +450,11 @@ def _auto_num_splits(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, h
 
 def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits: int = 0, max_seqlen_k: int = 0,
                       cu_seqlens_q=None, max_seqlen_q: int = 0, scale: float = 0.0, mask_type: int = MASK_NONE,
-                      window=(-1, -1), workspace=None, out=None) -> torch.Tensor:
-    """Paged decode = split-KV forward + LSE combine; num_splits = 0 asks the heuristic (needs max_seqlen_k)."""
+                      window=(-1, -1), workspace=None, out=None, fused: bool = False) -> torch.Tensor:
+    """Paged decode = split-KV forward + LSE combine; num_splits = 0 asks the heuristic (needs max_seqlen_k).
+
+    fused = True runs both in one launch that allocates nothing (fmha_fwd_splitkv_fused; the partial results then live
+    in the library's fixed device array, `workspace` is not used, and problems beyond its limits raise)."""
     group = cu_seqlens_q is not None
     _check_tensor("q", q, ndim=3 if group else 4)
     _check_tensor("k_cache", k_cache, dtype=q.dtype, ndim=4)
@@ -407,6 +474,10 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * k_cache.shape[1]
         num_splits = _auto_num_splits(B, Hq, Hk, sq, max_seqlen_k, D, k_cache.shape[1], q.dtype)
+    if fused:
+        return fmha_fwd_splitkv_fused(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_k, block_table=block_table,
+                                      cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, scale=scale,
+                                      mask_type=mask_type, window=window, out=out)
     o_acc, lse_acc = workspace if workspace is not None else (None, None)
     o_acc, lse_acc = fmha_fwd_splitkv(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_k, block_table=block_table,
                                       cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, scale=scale,

@@ -98,6 +98,32 @@ FCK_EXPORT int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v,
                                     void* stream);
 
 /*
+ * Split-KV forward and LSE combine in ONE launch that allocates nothing: fck_fmha_fwd_splitkv with `o` in place of
+ * the (lse_acc, o_acc) workspace.  It has no counterpart in the reference (whose callers always own the workspace and
+ * launch FmhaFwdSplitKV and FmhaFwdSplitKVCombine separately); it is for callers that cannot allocate or want a single
+ * launch: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ *
+ * The partial results go to a fixed device array inside the library (one copy per GPU, 16 MiB + 64 KiB, held until
+ * the process ends) and the workgroup that delivers the last partial result of a (sequence, KV-head group) merges
+ * the splits and writes `o`.  Limits: Bs * Hq * num_splits * Sq * (Dv + 1) <= 4 Mi floats and
+ * B * Hk * row_tiles <= 16384, else FCK_ERR_UNSUPPORTED (nothing is launched).  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams, different threads) race; calls on one stream are safe.
+ *
+ * num_splits > 0: that many equal key ranges, exactly as fck_fmha_fwd_splitkv.  num_splits == 0: the library takes
+ * fck_fmha_num_splits_heuristic of the CU count and the longest possible KV length (the block table's capacity, else
+ * seqlen_k).  The other arguments are those of fck_fmha_fwd_splitkv.
+ */
+FCK_EXPORT int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, const void* bias, void* o,
+                                          const int32_t* seqstart_q, const int32_t* seqstart_k,
+                                          const int32_t* seqlen_k_ptr, const int32_t* block_table,
+                                          const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
+                                          int64_t seqlen_k, int64_t q_num_heads, int64_t kv_num_heads,
+                                          int64_t qk_head_dim, int64_t v_head_dim, int64_t q_max_seq_len,
+                                          int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size,
+                                          float scale, int64_t window_left, int64_t window_right, uint32_t mask_type,
+                                          int32_t dtype, void* stream);
+
+/*
  * LSE combine: O = sum_s exp(lse_acc[s] - logsumexp_s lse_acc) * o_acc[s], stored as T.
  * Replaces `FmhaSplitKVCombine` / `FmhaFwdSplitKVCombine`, fmha_fwd_split_kv_combine_jinja.h:78-92
  * (args :37-76, strides :114-165), declared at fmha_fwd_split_kv_combine_call.h:26-36.

@@ -79,6 +79,17 @@ def test_paged_decode_head_pairs(fmha, orc, dtype, d, page):
     _run_paged(fmha, orc, kv, 4, mask_type=2, window=(40, 0))  # sliding window: leading tiles are skipped
 
 
+def test_decode_paged_fused_flag(fmha, orc):
+    """fmha_decode_paged(fused=True) = one launch; same result as the two-launch path within the output tolerance."""
+    w = gen.workload_paged_decode(seed=91, batch=5, hq=32, hk=8, head_dim=128, min_len=1, max_len=3000)
+    args = (dev(w["q"]), dev(w["k_cache"]), dev(w["v_cache"]), dev(w["seqlen_k"]), dev(w["block_table"]))
+    o1 = fmha.fmha_decode_paged(*args, num_splits=0, max_seqlen_k=3000, scale=w["scale"], fused=True)
+    o2 = fmha.fmha_decode_paged(*args, num_splits=0, max_seqlen_k=3000, scale=w["scale"])
+    ro = orc.fmha_fwd(w["q"], w["k_cache"], w["v_cache"], seqlen_k=w["seqlen_k"], block_table=w["block_table"], scale=w["scale"])
+    assert_close(o1, ro, 2e-2, "fused")
+    assert_close(o2, ro, 2e-2, "two launches")
+
+
 def test_group_mode_ragged_queries(fmha, orc):
     # ragged query counts (1..16 new tokens per sequence) through seqstart_q
     g = torch.Generator().manual_seed(5)

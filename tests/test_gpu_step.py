@@ -120,8 +120,9 @@ def test_page_size_one(fmha, orc):
     assert_close(od, rd, 2e-2, "decode, page size 1")
 
 
-def test_decode_captured_in_a_graph(fmha, orc, fused=False):
-    """A decode launch sequence (appendKV + split-KV + combine) captured into a HIP
+@pytest.mark.parametrize("fused", [False, True])
+def test_decode_captured_in_a_graph(fmha, orc, fused):
+    """A decode launch sequence (appendKV + split-KV + combine, or appendKV + the fused launch) captured into a HIP
     graph after one eager warm-up call, then replayed three times with new inputs written into the captured buffers and
     eager work and synchronisations between the replays; every replay is checked against the oracle.  The operators
     enqueue kernels only (no memset, no allocation), so the capture holds nothing else."""
@@ -142,7 +143,7 @@ def test_decode_captured_in_a_graph(fmha, orc, fused=False):
         fmha.fmha_fwd_appendkv(q, kc, vc, knew, vnew, sl, rotary_cos=dcos, rotary_sin=dsin, rope_mode=fmha.ROPE_HALF_ROTATED,
                                block_table=bt)
         torch.add(sl, 1, out=sl_after)
-        fmha.fmha_decode_paged(q, kc, vc, sl_after, bt, num_splits=3, workspace=ws, out=out)
+        fmha.fmha_decode_paged(q, kc, vc, sl_after, bt, num_splits=3, workspace=None if fused else ws, out=out, fused=fused)
 
     def new_inputs():
         hq_, hk_ = gen.randn((B, 1, hq, d), torch.bfloat16, g), gen.randn((B, 1, hk, d), torch.bfloat16, g)
