@@ -332,14 +332,20 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t
     // The direct-to-LDS kernels address a tile's rows with 32-bit byte offsets from the tile's first row.
     if ((int64_t)a.hk * d * 2 * 64 >= ((int64_t)1 << 31))
         return fail(FCK_ERR_INVALID_ARGUMENT, "kv_num_heads * head_dim = %ld is too large (64 cache rows must span < 2 GiB)", (long)(a.hk * d));
-    // Long query runs at head dim <= 128 take the 8-wave ping-pong kernel (256 rows per workgroup); short runs and
-    // head dim 256 take the 4-wave kernel (128 rows per workgroup).
+    // Long query runs at head dim <= 128 take the 8-wave ping-pong kernel (256 rows per workgroup).  Head dim 256
+    // takes the 4-wave kernel that sends K/V tiles straight to LDS (128 rows per workgroup) when a 64-key tile never
+    // straddles a page; short runs at head dim <= 128 and page sizes that are not a multiple of 64 take the 4-wave
+    // kernel that stages K/V through registers.
     if (d <= 128 && q_max_seq_len > 128) {
         a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
         g_kernel = uniform ? "prefill_pp_kernel<uniform_page>" : "prefill_pp_kernel<row_lookup>";
         return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }
     a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
+    if (d == 256 && uniform) {
+        g_kernel = "prefill_dma_kernel<uniform_page>";
+        return launch_status(fck::launch_prefill_dma(a, (int)d, dtype, static_cast<hipStream_t>(stream)), what);
+    }
     g_kernel = uniform ? "prefill_kernel<uniform_page>" : "prefill_kernel<row_lookup>";
     return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
 }

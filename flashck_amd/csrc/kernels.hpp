@@ -101,22 +101,15 @@ int splitkv_decode_m_tiles(int d, int rows_max);
 hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st);
 hipError_t launch_appendkv(const AppendKvArgs& a, int dtype, int max_new, hipStream_t st);
 hipError_t launch_prefill(const PrefillArgs& a, int d, int dtype, bool uniform_page, hipStream_t st);
-// Tiles of a sequence whose page ids the ping-pong prefill kernel caches in LDS; with more tiles than this the caller
-// must pass uniform_page = false (per-row table lookups).
+// Tiles of a sequence whose first rows the direct-to-LDS prefill kernels cache in LDS; tiles past them are looked up one
+// by one.
 constexpr int kPrefillPageCache = 4096;
 constexpr int kPrefillKeyTile = 64;
 // 256-row workgroups (a.m_tiles counts 256-row tiles); head dims 64 and 128
 hipError_t launch_prefill_pingpong(const PrefillArgs& a, int d, int dtype, bool uniform_page, hipStream_t st);
 
-// Streaming (persistent) variant of the ping-pong kernel: one workgroup per CU walks a list of work items.  Limits:
-// first rows of at most kPrefillStreamRowCache key tiles per item are cached (uniform_page rule as above with this
-// count), and a workgroup's list holds at most kPrefillStreamMaxItems items (prefill_stream_fits).
-constexpr int kPrefillStreamRowCache = 2048;
-constexpr int kPrefillStreamMaxItems = 1024;
 // Head dim 256 with the K/V tiles sent global -> LDS directly (128-row workgroups; a.m_tiles counts 128-row tiles);
-// uniform pages with at most kPrefillPageCache key tiles per sequence.
+// uniform pages only.
 hipError_t launch_prefill_dma(const PrefillArgs& a, int d, int dtype, hipStream_t st);
-bool prefill_stream_fits(const PrefillArgs& a, int num_cu);
-hipError_t launch_prefill_stream(const PrefillArgs& a, int d, int dtype, int num_cu, hipStream_t st);
 
 }  // namespace fck

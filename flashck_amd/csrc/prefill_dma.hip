@@ -10,8 +10,8 @@
 // LDS (a per-tile page-table load would sit on the critical path and drain the load queue each time).  The grid is 1-D in
 // XCD-aware order: all workgroups that stream one (sequence, KV head) run on one XCD, heaviest row tiles first.
 //
-// Limits: uniform pages only (page size a multiple of the 64-key tile, or no paging), at most kPrefillPageCache key
-// tiles per sequence; the launcher's caller falls back to prefill.hip otherwise.
+// Limits: uniform pages only (page size a multiple of the 64-key tile, or no paging; the caller takes prefill.hip
+// otherwise); the first rows of the first kPrefillPageCache key tiles are cached, later tiles are looked up one by one.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -77,25 +77,28 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
         q_row0 = b * a.sq;
         sq_b = a.sq;
     }
-    const int m0 = mt * S::BM;
-    if (m0 >= sq_b) return;
+    // Row tiles are aligned to the END of the sequence (the ragged tile is the first one, where a causal mask leaves
+    // the fewest keys): tile mt covers rows [mt * BM - pad, (mt + 1) * BM - pad), pad = (-sq) mod BM.
+    const int tiles_b = (sq_b + S::BM - 1) / S::BM;
+    if (mt >= tiles_b) return;
+    const int m0 = mt * S::BM - (tiles_b * S::BM - sq_b);  // negative for a ragged first tile
     const KvSeq ks = kv_seq(a.kv, b);
     const int sk_b = ks.len;
     const MaskYX mk = make_mask(a.mask_type, a.window_left, a.window_right, sq_b, sk_b);
 
     // this lane's query row
     const int r = m0 + wave * 32 + l32;
-    const bool row_ok = r < sq_b;
+    const bool row_ok = r >= 0 && r < sq_b;
     const int lo_r = row_ok ? mask_lo(mk, r) : 0;
     const int hi_r = row_ok ? mask_hi(mk, r, sk_b) : sk_b;
     // wave-uniform bounds: keys in [w_lo_max, w_hi_min) are visible to every valid row of the wave
-    const int wr0 = m0 + wave * 32;
-    const int wr1 = min(wr0 + 32, sq_b) - 1;
-    const bool wave_ok = wr0 < sq_b;
+    const int wr0 = max(m0 + wave * 32, 0);
+    const int wr1 = min(m0 + wave * 32 + 32, sq_b) - 1;
+    const bool wave_ok = wr1 >= wr0;
     const int w_lo_max = wave_ok ? mask_lo(mk, wr1) : 0;
     const int w_hi_min = wave_ok ? mask_hi(mk, wr0, sk_b) : sk_b;
     // workgroup-uniform visible range
-    const int t_begin = mask_lo(mk, m0) / BN;
+    const int t_begin = mask_lo(mk, max(m0, 0)) / BN;
     const int t_end = (mask_hi(mk, min(m0 + S::BM, sq_b) - 1, sk_b) + BN - 1) / BN;
     const int n = t_end - t_begin;  // number of tiles (may be <= 0)
 
@@ -150,6 +153,14 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     int row_vec = 0, row_chunk = -1;  // lane l: first row of tile row_chunk * 64 + l
     auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t {
         if (ks.table != nullptr) {
+            if (i >= kPrefillPageCache) {
+                // more key tiles than the cache holds (> kPrefillPageCache * 64 keys): one scalar table lookup per tile
+                const int kb = (t_begin + i) * BN;
+                const int pi = a.kv.page_shift >= 0 ? kb >> a.kv.page_shift : kb / a.kv.page_size;
+                int page = ((const __attribute__((address_space(4))) int32_t*)ks.table)[pi];
+                asm volatile("" : "+s"(page));
+                return (int64_t)page * a.kv.page_size + (kb - pi * a.kv.page_size);
+            }
             if ((i >> 6) != row_chunk) {
                 row_chunk = i >> 6;
                 row_vec = row_lds[min(row_chunk * 64 + lane, kPrefillPageCache - 1)];

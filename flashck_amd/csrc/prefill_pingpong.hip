@@ -110,25 +110,29 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         q_row0 = b * a.sq;
         sq_b = a.sq;
     }
-    const int m0 = mt * S::BM;
-    if (m0 >= sq_b) return;
+    // Row tiles are aligned to the END of the sequence: tile mt covers rows [mt * BM - pad, (mt + 1) * BM - pad) with
+    // pad = (-sq) mod BM, so the ragged tile is the first one.  Under a causal mask the first tile sees the fewest keys,
+    // so the rows that do not exist cost little there, and the last, most expensive tile is always full.
+    const int tiles_b = (sq_b + S::BM - 1) / S::BM;
+    if (mt >= tiles_b) return;
+    const int m0 = mt * S::BM - (tiles_b * S::BM - sq_b);  // negative for a ragged first tile
     const KvSeq ks = kv_seq(a.kv, b);
     const int sk_b = ks.len;
     const MaskYX mk = make_mask(a.mask_type, a.window_left, a.window_right, sq_b, sk_b);
 
     // this lane's query row
     const int r = m0 + group * 128 + wg * 32 + l32;
-    const bool row_ok = r < sq_b;
+    const bool row_ok = r >= 0 && r < sq_b;
     const int lo_r = row_ok ? mask_lo(mk, r) : 0;
     const int hi_r = row_ok ? mask_hi(mk, r, sk_b) : sk_b;
     // wave-uniform: keys in [w_lo_max, w_hi_min) are visible to every valid row of the wave
-    const int wr0 = m0 + group * 128 + wg * 32;
-    const bool wave_ok = wr0 < sq_b;
-    const int wr1 = min(wr0 + 32, sq_b) - 1;
+    const int wr0 = max(m0 + group * 128 + wg * 32, 0);
+    const int wr1 = min(m0 + group * 128 + wg * 32 + 32, sq_b) - 1;
+    const bool wave_ok = wr1 >= wr0;
     const int w_lo_max = wave_ok ? mask_lo(mk, wr1) : 0;
     const int w_hi_min = wave_ok ? mask_hi(mk, wr0, sk_b) : sk_b;
     // tiles the workgroup walks (a group also walks the few tiles only the other group can see: they mask to zero)
-    const int t_begin = mask_lo(mk, m0) / S::BN;
+    const int t_begin = mask_lo(mk, max(m0, 0)) / S::BN;
     const int t_end = (mask_hi(mk, min(m0 + S::BM, sq_b) - 1, sk_b) + S::BN - 1) / S::BN;
     const int n = t_end - t_begin;  // number of tiles (may be <= 0)
 

@@ -1,16 +1,6 @@
-"""GPU parity of the streaming (persistent-grid) prefill kernel against the CPU oracle.
-
-Two kernels are selected for a whole process by variables read once when the library takes its first prefill call:
-the streaming kernel by FLASHCK_PREFILL_STREAM=1 (first part of this file), the direct-to-LDS head-dim-256 kernel by
-FLASHCK_PREFILL_DMA256=1 (second part).  Neither has run on a GPU yet, so without its variable a test here is skipped;
-with it
-
-    FLASHCK_PREFILL_STREAM=1 python -m pytest tests/test_gpu_stream.py tests/test_gpu_prefill.py -m gpu
-
-runs them and sends every long-query prefill of the regular suite through the same kernel.
-"""
-import os
-
+"""GPU parity of the direct-to-LDS prefill kernels against the CPU oracle on workloads with many workgroups per CU:
+several row tiles and heads per sequence, mixed lengths, every mask kind, repeated launches; head dims 64 / 128
+(ping-pong kernel) and 256 (4-wave direct-to-LDS kernel)."""
 import pytest
 import torch
 
@@ -18,8 +8,6 @@ from flashck_amd import generators as gen
 from helpers import ATOL, assert_close, dev
 
 pytestmark = pytest.mark.gpu
-stream = pytest.mark.skipif(os.environ.get("FLASHCK_PREFILL_STREAM") != "1",
-                            reason="the streaming prefill kernel has not run on a GPU yet; set FLASHCK_PREFILL_STREAM=1")
 
 
 def _check(fmha, orc, w, dtype, what):
@@ -32,30 +20,26 @@ def _check(fmha, orc, w, dtype, what):
     assert_close(o, ro, ATOL[dtype], what)
 
 
-@stream
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("page", [64, 128])
 def test_few_items_per_workgroup(fmha, orc, dtype, d, page):
-    # 5 sequences x 4 heads x at most 2 row tiles: every workgroup gets at most one item (cold start and drain only)
+    # 5 sequences x 4 heads x at most 2 row tiles
     w = gen.workload_varlen_prefill(seed=150 + d + page, batch=5, hq=4, hk=2, head_dim=d, min_len=129, max_len=400,
                                     page_size=page, dtype=dtype)
-    _check(fmha, orc, w, dtype, "one item per workgroup")
+    _check(fmha, orc, w, dtype, "few workgroups")
 
 
-@stream
 @pytest.mark.parametrize("d", [64, 128])
 def test_many_items_per_workgroup(fmha, orc, d):
-    # 48 sequences x 16 heads x up to 5 row tiles on 256 workgroups: several items each, hand-offs between items of at
-    # least four tiles, cold starts after the short ones (lengths from 130 rows = 3 tiles up)
+    # 48 sequences x 16 heads x up to 5 row tiles: several workgroups per CU (lengths from 130 rows = 3 key tiles up)
     w = gen.workload_varlen_prefill(seed=160 + d, batch=48, hq=16, hk=4, head_dim=d, min_len=130, max_len=1200,
                                     page_size=64, dtype=torch.bfloat16)
-    _check(fmha, orc, w, torch.bfloat16, "several items per workgroup")
+    _check(fmha, orc, w, torch.bfloat16, "many workgroups")
 
 
-@stream
 def test_short_and_long_sequences_mixed(fmha, orc):
-    # one-tile and two-tile items (never handed off to) between long ones, one max_seqlen_q far above most lengths
+    # one-tile and two-tile sequences between long ones, max_seqlen_q far above most lengths
     g = torch.Generator().manual_seed(170)
     lens = [1, 2000, 63, 64, 65, 1500, 129, 257, 700, 130, 5, 1999]
     w = gen.workload_varlen_prefill(seed=170, batch=len(lens), hq=8, hk=8, head_dim=128, min_len=1, max_len=2000,
@@ -63,7 +47,6 @@ def test_short_and_long_sequences_mixed(fmha, orc):
     _check(fmha, orc, w, torch.bfloat16, "mixed lengths")
 
 
-@stream
 @pytest.mark.parametrize("mask", [(0, (-1, -1)), (2, (-1, 0)), (2, (100, 0)), (1, (-1, 0))])
 def test_dense_batch_mode_masks(fmha, orc, mask):
     # no page table: contiguous K/V, every mask kind, sliding window (row tiles that start past tile 0)
@@ -74,10 +57,9 @@ def test_dense_batch_mode_masks(fmha, orc, mask):
     mt, win = mask
     o = fmha.fmha_fwd(dev(q), dev(k), dev(v), mask_type=mt, window=win)
     ro = orc.fmha_fwd(q, k, v, mask_type=mt, window=win)
-    assert_close(o, ro, 2e-2, "dense, streamed")
+    assert_close(o, ro, 2e-2, "dense, masks")
 
 
-@stream
 def test_repeated_launches_agree(fmha, orc):
     # the kernel keeps no state between launches: the same call twice gives the same bits
     w = gen.workload_varlen_prefill(seed=190, batch=20, hq=8, hk=2, head_dim=128, min_len=200, max_len=900, page_size=128)
@@ -87,15 +69,8 @@ def test_repeated_launches_agree(fmha, orc):
     assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
 
 
-# ---------------------------------------------------------------------------------------------------------------------
-# The direct-to-LDS head-dim-256 kernel (FLASHCK_PREFILL_DMA256=1): same status, same way to run it:
-#     FLASHCK_PREFILL_DMA256=1 python -m pytest tests/test_gpu_stream.py tests/test_gpu_prefill.py -m gpu -k "256 or dma"
-# ---------------------------------------------------------------------------------------------------------------------
-dma256 = pytest.mark.skipif(os.environ.get("FLASHCK_PREFILL_DMA256") != "1",
-                            reason="the direct-to-LDS head-dim-256 kernel has not run on a GPU yet; set FLASHCK_PREFILL_DMA256=1")
 
-
-@dma256
+# ---- head dim 256 ----
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("page", [64, 128])
 def test_dma256_paged(fmha, orc, dtype, page):
@@ -104,7 +79,6 @@ def test_dma256_paged(fmha, orc, dtype, page):
     _check(fmha, orc, w, dtype, "head dim 256, direct to LDS")
 
 
-@dma256
 @pytest.mark.parametrize("mask", [(0, (-1, -1)), (2, (-1, 0)), (2, (90, 0)), (1, (-1, 0))])
 def test_dma256_dense_masks(fmha, orc, mask):
     g = torch.Generator().manual_seed(260)
