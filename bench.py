@@ -21,11 +21,30 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
 
-# HBM bytes one split-KV launch of the default workload moves, from two counter runs of this script
-# (`rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --no-extra --no-cpu --steps 20 --warmup 5`, then WRITE_SIZE):
-# 262,504.5 KiB fetched and 1,088 KiB written per dispatch, each scaled by what the same counter reads for a 512 MiB
-# device copy (`--workload copy`: FETCH_SIZE reads half the bytes copied -> x2.0, WRITE_SIZE reads them all -> x1.0).
-SPLITKV_DEFAULT_TRAFFIC_BYTES = int(262504.5 * 1024 * 2.0 + 1088 * 1024 * 1.0)
+COUNTER_FILE = os.path.join(ROOT, "profiles", "splitkv_decode_cfg3.md")
+DECODE_SOURCE = os.path.join(ROOT, "flashck_amd", "csrc", "splitkv_decode.hip")
+
+
+def measured_traffic(kernel):
+    """HBM bytes one split-KV launch of the default workload moved when the hardware counters were last read, or None.
+
+    The figure is not measured by this run: it comes from the `counters` line of profiles/splitkv_decode_cfg3.md (two
+    `rocprofv3 --pmc` runs of this script, FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same
+    counter reads for a plain device copy of known size).  It is only reported while it still describes the code that
+    runs: same kernel variant and same source file as when the counters were read.
+    """
+    import hashlib
+    import re
+    try:
+        text = open(COUNTER_FILE).read()
+        sha = hashlib.sha256(open(DECODE_SOURCE, "rb").read()).hexdigest()
+    except OSError:
+        return None
+    m = re.search(r'counters kernel="([^"]+)" source_sha256=([0-9a-f]+) fetch_kib=([0-9.]+) write_kib=([0-9.]+) '
+                  r'fetch_scale=([0-9.]+) write_scale=([0-9.]+)', text)
+    if not m or m.group(1) != kernel or m.group(2) != sha:
+        return None
+    return int(float(m.group(3)) * 1024 * float(m.group(5)) + float(m.group(4)) * 1024 * float(m.group(6)))
 
 
 def parse():
@@ -83,6 +102,7 @@ def time_steps(fn, steps, warmup, torch, kernel_events=False):
 
 
 def bench_decode(args, torch, fmha, gen, which):
+    from flashck_amd import _lib
     if which == "splitkv":
         w = gen.workload_splitkv_decode(kv_len=args.kv_len, num_splits=args.num_splits, shuffle=not args.no_shuffle)
         ns = w["num_splits"]
@@ -127,11 +147,12 @@ def bench_decode(args, torch, fmha, gen, which):
             fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, out=o)
 
     wall, kern_ms = time_steps(step, args.steps, args.warmup, torch, kernel_events="region" if fused else True)
+    kernel = _lib.load().fck_fmha_last_kernel().decode()  # the combine launch does not change it
     nbytes = gen.decode_bytes(w["lens"], [1] * B, Hq, Hk, D, D, 128)
     flops = gen.decode_flops(w["lens"], [1] * B, Hq, D, D)
     ms = wall / args.steps * 1e3
     res = dict(name=name, ms_per_step=ms, bytes=nbytes, flops=flops, gbs=nbytes / (ms * 1e-3) / 1e9,
-               kernel_ms=kern_ms, kernel_gbs=nbytes / (kern_ms * 1e-3) / 1e9, num_splits=ns, w=w)
+               kernel_ms=kern_ms, kernel_gbs=nbytes / (kern_ms * 1e-3) / 1e9, num_splits=ns, w=w, kernel=kernel)
     return res
 
 
@@ -149,12 +170,14 @@ def bench_prefill(args, torch, fmha, gen, d, steps, warmup):
             ev[1].record()
 
     wall, kern_ms = time_steps(step, steps, warmup, torch, kernel_events=True)
+    from flashck_amd import _lib
+    kernel = _lib.load().fck_fmha_last_kernel().decode()
     flops = gen.prefill_flops(w["lens"], 32, d, d)
     nbytes = gen.prefill_bytes(w["lens"], 32, 8, d, d)
     ms = wall / steps * 1e3
     return dict(name=f"varlen causal batch prefill: 16 seqs L~U[128,8192] Hq32/Hk8 D{d} paged P=128 (bf16)",
                 ms_per_step=ms, flops=flops, bytes=nbytes, tflops=flops / (ms * 1e-3) / 1e12, kernel_ms=kern_ms,
-                kernel_tflops=flops / (kern_ms * 1e-3) / 1e12, total_q=sum(w["lens"]))
+                kernel_tflops=flops / (kern_ms * 1e-3) / 1e12, total_q=sum(w["lens"]), kernel=kernel)
 
 
 def bench_appendkv(args, torch, fmha, gen, steps, warmup):
@@ -224,9 +247,10 @@ def main():
     if args.workload in ("splitkv", "paged_decode"):
         r = bench_decode(args, torch, fmha, gen, args.workload)
         value, unit, metric = r["gbs"], "GB/s", "paged-KV decode HBM GB/s (% of peak) + us/call; prefill TFLOP/s, MFMA util %"
-        default_shape = args.workload == "splitkv" and args.kv_len == 32768 and args.num_splits == 8 and not args.no_shuffle
-        traffic = SPLITKV_DEFAULT_TRAFFIC_BYTES if default_shape else None  # counters were only read for that shape
-        roof = dict(bound="hbm", kernel="splitkv_decode_kernel", achieved=r["kernel_gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
+        default_shape = (args.workload == "splitkv" and args.kv_len == 32768 and args.num_splits == 8 and not args.no_shuffle
+                         and args.decode_path == "two-launch")
+        traffic = measured_traffic(r["kernel"]) if default_shape else None  # counters were only read for that shape
+        roof = dict(bound="hbm", kernel=r["kernel"], achieved=r["kernel_gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=r["kernel_gbs"] / HBM_PEAK_GBS, traffic=traffic, bytes_per_launch=r["bytes"],
                     avg_launch_us=r["kernel_ms"] * 1e3)
         extra["pct_of_hbm_peak"] = 100.0 * value / HBM_PEAK_GBS
@@ -242,7 +266,7 @@ def main():
         d = 128 if args.workload == "prefill" else 256
         r = bench_prefill(args, torch, fmha, gen, d, args.steps, args.warmup)
         value, unit, metric = r["tflops"], "TFLOP/s", "varlen causal prefill TFLOP/s (MFMA util %)"
-        roof = dict(bound="mfma", kernel="prefill_pp_kernel" if d == 128 else "prefill_kernel", achieved=r["kernel_tflops"], peak=MFMA_BF16_PEAK_TFLOPS,
+        roof = dict(bound="mfma", kernel=r["kernel"], achieved=r["kernel_tflops"], peak=MFMA_BF16_PEAK_TFLOPS,
                     unit="TFLOP/s", frac=r["kernel_tflops"] / MFMA_BF16_PEAK_TFLOPS, traffic=None,
                     flops_per_launch=r["flops"], avg_launch_us=r["kernel_ms"] * 1e3)
         cpu = None
@@ -271,8 +295,20 @@ def main():
         def prefill(d):
             r5 = bench_prefill(args, torch, fmha, gen, d, 10, 3)
             return dict(workload=r5["name"], ms_per_call=r5["ms_per_step"], tflops=r5["tflops"],
-                        mfma_util_pct=100 * r5["tflops"] / MFMA_BF16_PEAK_TFLOPS, flops=r5["flops"], kernel_ms=r5["kernel_ms"])
+                        mfma_util_pct=100 * r5["tflops"] / MFMA_BF16_PEAK_TFLOPS, flops=r5["flops"], kernel_ms=r5["kernel_ms"],
+                        kernel=r5["kernel"])
 
+        def splitkv_variant(path, ns):
+            a2 = argparse.Namespace(**vars(args))
+            a2.steps, a2.warmup, a2.decode_path, a2.num_splits = max(20, args.steps // 2), 10, path, ns
+            r3 = bench_decode(a2, torch, fmha, gen, "splitkv")
+            return dict(workload=r3["name"], us_per_call=r3["ms_per_step"] * 1e3, gbs=r3["gbs"],
+                        pct_of_hbm_peak=100 * r3["gbs"] / HBM_PEAK_GBS, kernel_us=r3["kernel_ms"] * 1e3, num_splits=r3["num_splits"])
+
+        # the same workload with the split count the library's heuristic picks, and as one fused launch
+        ns_lib = fmha.num_splits_heuristic(4, 64, 8, 1, args.kv_len, 128)
+        secondary("splitkv_library_splits", lambda: splitkv_variant("two-launch", ns_lib))
+        secondary("splitkv_fused", lambda: splitkv_variant("fused", 0))
         secondary("paged_decode", paged)
         secondary("appendkv", append)
         for d in (128, 256):
