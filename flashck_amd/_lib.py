@@ -12,12 +12,25 @@ LIB_PATH = os.environ.get("FLASHCK_FMHA_LIB") or os.path.join(_HERE, "libflashck
 
 _vp, _i64, _i32, _u32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_uint32, ctypes.c_float
 
+class Attrs(ctypes.Structure):
+    """fck_fmha_attrs of the header."""
+    _fields_ = [("size", ctypes.c_uint32), ("bias_type", ctypes.c_int32), ("bias", ctypes.c_void_p),
+                ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64),
+                ("logits_soft_cap", ctypes.c_float), ("reserved", ctypes.c_uint32)]
+
+
+_ap = ctypes.POINTER(Attrs)
+
 # name -> (restype, argtypes); order and types follow the header
 SIGNATURES = {
     "fck_last_error": (ctypes.c_char_p, []),
     "fck_fmha_version": (ctypes.c_char_p, []),
     "fck_fmha_last_kernel": (ctypes.c_char_p, []),
     "fck_fmha_fwd": (ctypes.c_int, [_vp] * 8 + [_i64] * 8 + [_f32, _i64, _i64, _u32, _i32, _vp]),
+    "fck_fmha_fwd_attrs": (ctypes.c_int, [_vp] * 8 + [_i64] * 8 + [_f32, _i64, _i64, _u32, _i32, _ap, _vp]),
+    "fck_fmha_fwd_splitkv_attrs": (ctypes.c_int, [_vp] * 11 + [_i64] * 11 + [_f32, _i64, _i64, _u32, _i32, _ap, _vp]),
+    "fck_fmha_batch_prefill_attrs": (ctypes.c_int, [_vp] * 8 + [_i64] * 8 + [_f32, _i64, _i64, _u32, _i32, _ap, _vp]),
+    "fck_fmha_fwd_pagedkv_attrs": (ctypes.c_int, [_vp] * 7 + [_i64] * 9 + [_f32, _i64, _i64, _u32, _i32, _ap, _vp]),
     "fck_fmha_fwd_splitkv": (ctypes.c_int, [_vp] * 11 + [_i64] * 11 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_fwd_splitkv_fused": (ctypes.c_int, [_vp] * 10 + [_i64] * 11 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_fwd_splitkv_combine": (ctypes.c_int, [_vp] * 4 + [_i64] * 6 + [_i32, _vp]),

@@ -237,6 +237,91 @@ __host__ __device__ inline int32_t mask_hi(const MaskYX& m, int32_t i, int32_t s
     return v < sk ? (v > 0 ? (int32_t)v : 0) : sk;
 }
 
+// Optional score modifiers; an all-zero struct means none.  Order (ck_tile/ops/fmha/pipeline/
+// block_fmha_pipeline_qr_ks_vs.hpp:391-449): x = scale * q.k; soft cap x = cap * tanh(x / cap)
+// (ck_tile/ops/fmha/block/variants.hpp:208-209); bias added; then the mask.
+//   elementwise bias: data dtype, element (b, h, i, j) at bias[b * batch_stride + h * head_stride + i * row_stride + j]
+//                     (group mode: i counts from the first packed query row of the sequence, batch_stride unused):
+//                     ck_tile/ops/fmha/kernel/fmha_fwd_splitkv_kernel.hpp:608-688,925-932
+//   ALiBi:            fp32 slope of (b, h) at bias[b * batch_stride + h]; added term and mode as in
+//                     ck_tile/ops/fmha/block/block_position_encoding.hpp:19-121,138-152 and
+//                     ck_tile/ops/fmha/kernel/fmha_fwd_kernel.hpp:1482-1507
+struct ScoreMod {
+    const void* bias;
+    int64_t batch_stride, head_stride, row_stride;
+    int32_t bias_type;  // 0 none, 1 elementwise, 2 ALiBi
+    float soft_cap;     // > 0: on
+    float scale;        // the softmax scale in natural units (the soft cap is not linear, so it cannot be folded)
+    __host__ __device__ bool active() const { return bias_type != 0 || soft_cap > 0.f; }
+};
+
+// ALiBi position modes (AlibiMode, block_position_encoding.hpp:38-43)
+enum : int32_t { kAlibiVertical = 0, kAlibiTopLeft = 1, kAlibiBottomRight = 2 };
+
+// mode of a problem: a causal window (left < 0, right == 0) under any mask type gives VERTICAL, otherwise the mask type
+// names the diagonal; without a mask the diagonal ends at the bottom right corner
+__host__ __device__ inline int32_t alibi_mode(uint32_t mask_type, int64_t wl, int64_t wr)
+{
+    if (mask_type == 0) return kAlibiBottomRight;
+    if (wl < 0 && wr == 0) return kAlibiVertical;
+    return mask_type == 1 ? kAlibiTopLeft : kAlibiBottomRight;
+}
+
+__device__ __forceinline__ float fast_tanh(float x)
+{
+    // 1 - 2 / (e^(2x) + 1): exact limits at +-inf, relative error of a few ulp elsewhere
+    const float e = __builtin_amdgcn_exp2f(x * (2.f * kLog2e));
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+}
+
+// The modifiers of one query row, set up once per row; score() maps a raw dot product to the log2-domain score
+// (already multiplied by log2 e, so the caller's scale factor is 1).
+template <typename T>
+struct RowMod {
+    const uint16_t* bias_row;  // elementwise: row (b, h, i) of the bias
+    float slope;               // ALiBi: signed slope (positive for VERTICAL, negative otherwise)
+    int32_t zero;              // ALiBi: column of distance 0 (unused for VERTICAL)
+    int32_t mode;
+    int32_t last_key;          // bias reads are clamped to the row's last key
+    float scale, cap, cap_rcp;
+    int32_t bias_type;
+
+    __device__ __forceinline__ void init(const ScoreMod& m, int b, int64_t first_row, int h, int i, int sq, int sk, uint32_t mask_type,
+                                         int64_t wl, int64_t wr, bool group)
+    {
+        bias_type = m.bias_type;
+        scale = m.scale;
+        cap = m.soft_cap;
+        cap_rcp = m.soft_cap > 0.f ? 1.f / m.soft_cap : 0.f;
+        last_key = sk - 1;
+        bias_row = nullptr;
+        slope = 0.f;
+        zero = 0;
+        mode = alibi_mode(mask_type, wl, wr);
+        if (m.bias_type == 1) {
+            const int64_t brow = (group ? first_row : 0) + i;
+            bias_row = reinterpret_cast<const uint16_t*>(m.bias) + (group ? 0 : (int64_t)b * m.batch_stride) + (int64_t)h * m.head_stride +
+                       brow * m.row_stride;
+        } else if (m.bias_type == 2) {
+            const float sl = reinterpret_cast<const float*>(m.bias)[(int64_t)b * m.batch_stride + h];
+            slope = mode == kAlibiVertical ? sl : -sl;
+            zero = mode == kAlibiBottomRight ? i + sk - sq : i;
+        }
+    }
+    __device__ __forceinline__ float score(float qk, int key) const
+    {
+        float x = qk * scale;
+        if (cap > 0.f) x = cap * fast_tanh(x * cap_rcp);
+        if (bias_type == 1) {
+            x += T::to_f32(bias_row[min(max(key, 0), last_key)]);
+        } else if (bias_type == 2) {
+            const int dist = mode == kAlibiVertical ? key : abs(zero - key);
+            x = __builtin_fmaf(slope, (float)dist, x);
+        }
+        return x * kLog2e;
+    }
+};
+
 // Where the K/V rows of one sequence live.  `table` == nullptr: rows are contiguous from base_row.
 // Otherwise logical key j sits at row table[j / page] * page + j % page.
 struct KvSeq {

@@ -27,7 +27,7 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
-int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, int32_t dtype, const void* bias)
+int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, int32_t dtype)
 {
     if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16)
         return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
@@ -35,7 +35,50 @@ int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, i
     if (hq % hk != 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_num_heads %ld is not a multiple of kv_num_heads %ld", (long)hq, (long)hk);
     if (d != dv) return fail(FCK_ERR_UNSUPPORTED, "qk_head_dim %ld != v_head_dim %ld is not supported", (long)d, (long)dv);
     if (d != 64 && d != 128 && d != 256) return fail(FCK_ERR_UNSUPPORTED, "head_dim %ld: kernels exist for 64, 128, 256", (long)d);
-    if (bias) return fail(FCK_ERR_UNSUPPORTED, "attention bias / alibi is not supported");
+    return FCK_OK;
+}
+
+// Bias / ALiBi / soft cap of a call: `bias` is the positional pointer of the entry points that have one (else null).
+int fill_mod(fck::ScoreMod& m, const void* bias, const fck_fmha_attrs* at, float scale, uint32_t mask_type, int64_t hq)
+{
+    m = fck::ScoreMod{};
+    if (!at) {
+        if (bias) return fail(FCK_ERR_UNSUPPORTED, "a bias pointer needs the _attrs entry point: fck_fmha_attrs says what it holds");
+        return FCK_OK;
+    }
+    if (at->size != sizeof(fck_fmha_attrs))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "fck_fmha_attrs.size is %u, this library's struct has %zu bytes", at->size, sizeof(fck_fmha_attrs));
+    if (!bias) bias = at->bias;
+    if (at->bias && bias != at->bias) return fail(FCK_ERR_INVALID_ARGUMENT, "two different bias pointers (argument and fck_fmha_attrs.bias)");
+    if (!(at->logits_soft_cap >= 0.f) || !std::isfinite(at->logits_soft_cap))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "logits_soft_cap must be finite and >= 0 (0: off)");
+    switch (at->bias_type) {
+    case FCK_BIAS_NONE:
+        if (bias) return fail(FCK_ERR_INVALID_ARGUMENT, "a bias pointer with bias_type NO_BIAS");
+        break;
+    case FCK_BIAS_ELEMENTWISE:
+        if (!bias) return fail(FCK_ERR_INVALID_ARGUMENT, "bias_type ELEMENTWISE_BIAS needs a bias pointer");
+        if (reinterpret_cast<uintptr_t>(bias) & 1u) return fail(FCK_ERR_INVALID_ARGUMENT, "the bias must be 2-byte aligned");
+        if (at->bias_row_stride <= 0 || at->bias_head_stride < 0 || at->bias_batch_stride < 0)
+            return fail(FCK_ERR_INVALID_ARGUMENT, "elementwise bias: row stride must be positive, head and batch strides >= 0");
+        break;
+    case FCK_BIAS_ALIBI:
+        if (!bias) return fail(FCK_ERR_INVALID_ARGUMENT, "bias_type ALIBI needs the slopes pointer");
+        if (reinterpret_cast<uintptr_t>(bias) & 3u) return fail(FCK_ERR_INVALID_ARGUMENT, "ALiBi slopes are fp32: the pointer must be 4-byte aligned");
+        if (at->bias_batch_stride != 0 && at->bias_batch_stride < hq)
+            return fail(FCK_ERR_INVALID_ARGUMENT, "ALiBi: bias_batch_stride is 0 (slopes shared by all batches) or >= q_num_heads");
+        if (mask_type == FCK_MASK_GENERIC)
+            return fail(FCK_ERR_UNSUPPORTED, "ALiBi with mask_type GENERIC: the reference defines the diagonal for top-left and bottom-right only");
+        break;
+    default: return fail(FCK_ERR_INVALID_ARGUMENT, "bias_type %d out of range [0,2]", at->bias_type);
+    }
+    m.bias = bias;
+    m.bias_type = at->bias_type;
+    m.batch_stride = at->bias_batch_stride;
+    m.head_stride = at->bias_type == FCK_BIAS_ELEMENTWISE ? at->bias_head_stride : 0;
+    m.row_stride = at->bias_type == FCK_BIAS_ELEMENTWISE ? at->bias_row_stride : 0;
+    m.soft_cap = at->logits_soft_cap;
+    m.scale = scale;
     return FCK_OK;
 }
 
@@ -118,9 +161,9 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
                          const int32_t* block_table, const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
                          int64_t seqlen_k, int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len,
                          int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size, float scale,
-                         int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype)
+                         int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype, const fck_fmha_attrs* attrs)
 {
-    if (int rc = check_common(batch, hq, hk, d, dv, dtype, bias)) return rc;
+    if (int rc = check_common(batch, hq, hk, d, dv, dtype)) return rc;
     if (int rc = check_mask(mask_type)) return rc;
     if (!q || !k || !v) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k and v must not be null");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k and v must be 16-byte aligned");
@@ -147,6 +190,7 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
     a.mask_type = mask_type;
     a.window_left = window_left;
     a.window_right = window_right;
+    if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
 
     uniform = true;
     fck::KvAddr& kv = a.kv;
@@ -183,19 +227,33 @@ int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v, const void
                          int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size, float scale,
                          int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream)
 {
+    return fck_fmha_fwd_splitkv_attrs(q, k, v, bias, lse_acc, o_acc, seqstart_q, seqstart_k, seqlen_k_ptr, block_table, cache_batch_idx,
+                                      batch, seqlen_q, seqlen_k, hq, hk, d, dv, q_max_seq_len, num_splits, max_num_page_blocks,
+                                      page_block_size, scale, window_left, window_right, mask_type, dtype, nullptr, stream);
+}
+
+int fck_fmha_fwd_splitkv_attrs(const void* q, const void* k, const void* v, const void* bias, void* lse_acc, void* o_acc,
+                               const int32_t* seqstart_q, const int32_t* seqstart_k, const int32_t* seqlen_k_ptr,
+                               const int32_t* block_table, const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
+                               int64_t seqlen_k, int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len,
+                               int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size, float scale,
+                               int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype,
+                               const fck_fmha_attrs* attrs, void* stream)
+{
     g_err[0] = 0;
     fck::SplitKvArgs a;
     bool uniform;
     int rows_max;
     if (int rc = splitkv_setup(a, uniform, rows_max, q, k, v, bias, seqstart_q, seqstart_k, seqlen_k_ptr, block_table,
                                cache_batch_idx, batch, seqlen_q, seqlen_k, hq, hk, d, dv, q_max_seq_len, num_splits,
-                               max_num_page_blocks, page_block_size, scale, window_left, window_right, mask_type, dtype))
+                               max_num_page_blocks, page_block_size, scale, window_left, window_right, mask_type, dtype, attrs))
         return rc;
     if (!lse_acc || !o_acc) return fail(FCK_ERR_INVALID_ARGUMENT, "lse_acc and o_acc must not be null");
     if (!aligned16(o_acc)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_acc must be 16-byte aligned");
     a.o_acc = static_cast<float*>(o_acc);
     a.lse_acc = static_cast<float*>(lse_acc);
-    g_kernel = uniform ? "splitkv_decode_kernel<uniform_page>" : "splitkv_decode_kernel<row_lookup>";
+    g_kernel = a.mod.active() ? (uniform ? "splitkv_decode_kernel<uniform_page,score_mod>" : "splitkv_decode_kernel<row_lookup,score_mod>")
+                              : (uniform ? "splitkv_decode_kernel<uniform_page>" : "splitkv_decode_kernel<row_lookup>");
     return launch_status(fck::launch_splitkv_decode(a, (int)d, dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
                          "FmhaFwdSplitKV launch");
 }
@@ -220,7 +278,7 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
     int rows_max;
     if (int rc = splitkv_setup(a, uniform, rows_max, q, k, v, bias, seqstart_q, seqstart_k, seqlen_k_ptr, block_table,
                                cache_batch_idx, batch, seqlen_q, seqlen_k, hq, hk, d, dv, q_max_seq_len, num_splits,
-                               max_num_page_blocks, page_block_size, scale, window_left, window_right, mask_type, dtype))
+                               max_num_page_blocks, page_block_size, scale, window_left, window_right, mask_type, dtype, nullptr))
         return rc;
     if (!o) return fail(FCK_ERR_INVALID_ARGUMENT, "o must not be null");
     if (!aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "o must be 16-byte aligned");
@@ -336,6 +394,12 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t
     // takes the 4-wave kernel that sends K/V tiles straight to LDS (128 rows per workgroup) when a 64-key tile never
     // straddles a page; short runs at head dim <= 128 and page sizes that are not a multiple of 64 take the 4-wave
     // kernel that stages K/V through registers.
+    if (a.mod.active()) {
+        // bias, ALiBi and the soft cap are applied by the register-staged kernel only
+        a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
+        g_kernel = uniform ? "prefill_kernel<uniform_page,score_mod>" : "prefill_kernel<row_lookup,score_mod>";
+        return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+    }
     if (d <= 128 && q_max_seq_len > 128) {
         a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
         g_kernel = uniform ? "prefill_pp_kernel<uniform_page>" : "prefill_pp_kernel<row_lookup>";
@@ -355,8 +419,17 @@ int fck_fmha_fwd(const void* q, const void* k, const void* v, const void* bias, 
                  int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left,
                  int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream)
 {
+    return fck_fmha_fwd_attrs(q, k, v, bias, o, seqstart_q, seqstart_k, seqlen_k_ptr, batch, seqlen_q, seqlen_k, hq, hk, d, dv,
+                              q_max_seq_len, scale, window_left, window_right, mask_type, dtype, nullptr, stream);
+}
+
+int fck_fmha_fwd_attrs(const void* q, const void* k, const void* v, const void* bias, void* o, const int32_t* seqstart_q,
+                       const int32_t* seqstart_k, const int32_t* seqlen_k_ptr, int64_t batch, int64_t seqlen_q, int64_t seqlen_k,
+                       int64_t hq, int64_t hk, int64_t d, int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left,
+                       int64_t window_right, uint32_t mask_type, int32_t dtype, const fck_fmha_attrs* attrs, void* stream)
+{
     g_err[0] = 0;
-    if (int rc = check_common(batch, hq, hk, d, dv, dtype, bias)) return rc;
+    if (int rc = check_common(batch, hq, hk, d, dv, dtype)) return rc;
     if (int rc = check_mask(mask_type)) return rc;
     if (!q || !k || !v || !o) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v and o must not be null");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v and o must be 16-byte aligned");
@@ -376,6 +449,7 @@ int fck_fmha_fwd(const void* q, const void* k, const void* v, const void* bias, 
     a.mask_type = mask_type;
     a.window_left = window_left;
     a.window_right = window_right;
+    if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
     a.kv.page_shift = -1;
     a.kv.seqlen_k_ptr = seqlen_k_ptr;  // group mode: logical key counts of padded packed sequences
     if (seqstart_q) {
@@ -396,8 +470,19 @@ int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cac
                            int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left, int64_t window_right,
                            uint32_t mask_type, int32_t dtype, void* stream)
 {
+    return fck_fmha_batch_prefill_attrs(q, k_cache, v_cache, o, seqstart_q, kv_indptr, kv_page_indices, kv_last_page_lens,
+                                        num_total_pages, page_block_size, batch, hq, hk, d, dv, q_max_seq_len, scale, window_left,
+                                        window_right, mask_type, dtype, nullptr, stream);
+}
+
+int fck_fmha_batch_prefill_attrs(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
+                                 const int32_t* kv_indptr, const int32_t* kv_page_indices, const int32_t* kv_last_page_lens,
+                                 int64_t num_total_pages, int64_t page_block_size, int64_t batch, int64_t hq, int64_t hk,
+                                 int64_t d, int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left,
+                                 int64_t window_right, uint32_t mask_type, int32_t dtype, const fck_fmha_attrs* attrs, void* stream)
+{
     g_err[0] = 0;
-    if (int rc = check_common(batch, hq, hk, d, dv, dtype, nullptr)) return rc;
+    if (int rc = check_common(batch, hq, hk, d, dv, dtype)) return rc;
     if (int rc = check_mask(mask_type)) return rc;
     if (!q || !k_cache || !v_cache || !o || !seqstart_q || !kv_indptr || !kv_page_indices)
         return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, seqstart_q, kv_indptr and kv_page_indices must not be null");
@@ -417,6 +502,7 @@ int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cac
     a.mask_type = mask_type;
     a.window_left = window_left;
     a.window_right = window_right;
+    if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
     a.kv.mode = 3;
     a.kv.kv_indptr = kv_indptr;
     a.kv.kv_page_indices = kv_page_indices;
@@ -434,8 +520,19 @@ int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache
                          int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left, int64_t window_right,
                          uint32_t mask_type, int32_t dtype, void* stream)
 {
+    return fck_fmha_fwd_pagedkv_attrs(q, k_cache, v_cache, o, seqstart_q, seqlen_k_ptr, block_table, batch_stride_block_table,
+                                      page_block_size, batch, seqlen_q, hq, hk, d, dv, q_max_seq_len, scale, window_left, window_right,
+                                      mask_type, dtype, nullptr, stream);
+}
+
+int fck_fmha_fwd_pagedkv_attrs(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
+                               const int32_t* seqlen_k_ptr, const int32_t* block_table, int64_t batch_stride_block_table,
+                               int64_t page_block_size, int64_t batch, int64_t seqlen_q, int64_t hq, int64_t hk, int64_t d,
+                               int64_t dv, int64_t q_max_seq_len, float scale, int64_t window_left, int64_t window_right,
+                               uint32_t mask_type, int32_t dtype, const fck_fmha_attrs* attrs, void* stream)
+{
     g_err[0] = 0;
-    if (int rc = check_common(batch, hq, hk, d, dv, dtype, nullptr)) return rc;
+    if (int rc = check_common(batch, hq, hk, d, dv, dtype)) return rc;
     if (int rc = check_mask(mask_type)) return rc;
     if (!q || !k_cache || !v_cache || !o || !seqlen_k_ptr || !block_table)
         return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, seqlen_k and block_table must not be null");
@@ -457,6 +554,7 @@ int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache
     a.mask_type = mask_type;
     a.window_left = window_left;
     a.window_right = window_right;
+    if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
     a.kv.mode = 2;
     a.kv.block_table = block_table;
     a.kv.block_table_stride = (int32_t)batch_stride_block_table;

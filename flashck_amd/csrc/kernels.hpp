@@ -44,6 +44,7 @@ struct SplitKvArgs {
     float scale_log2;  // scale * log2(e)
     uint32_t mask_type;
     int64_t window_left, window_right;
+    ScoreMod mod;      // bias / ALiBi / soft cap; all zero: none
 };
 
 struct CombineArgs {
@@ -86,6 +87,7 @@ struct PrefillArgs {
     float scale_log2;
     uint32_t mask_type;
     int64_t window_left, window_right;
+    ScoreMod mod;  // bias / ALiBi / soft cap; all zero: none (only the 4-wave kernel of prefill.hip applies them)
 };
 
 hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page, int num_cu,

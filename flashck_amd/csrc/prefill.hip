@@ -33,7 +33,7 @@ constexpr size_t prefill_lds_bytes()
     return (size_t)4 * PrefillShape<D>::TILEB;
 }
 
-template <typename T, int D, bool kUniformPage>
+template <typename T, int D, bool kUniformPage, bool kMod = false>
 __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const PrefillArgs a)
 {
     typedef PrefillShape<D> S;
@@ -71,6 +71,11 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
     const bool row_ok = r < sq_b;
     const int lo_r = row_ok ? mask_lo(mk, r) : 0;
     const int hi_r = row_ok ? mask_hi(mk, r, sk_b) : sk_b;
+    // bias / ALiBi / soft cap of this lane's row; scores then come out in the log2 domain, so the scale becomes 1
+    RowMod<T> rmod;
+    if constexpr (kMod)
+        rmod.init(a.mod, b, q_row0, h, row_ok ? r : 0, sq_b, sk_b, a.mask_type, a.window_left, a.window_right, a.seqstart_q != nullptr);
+    const float scl = kMod ? 1.f : a.scale_log2;
     // wave-uniform bounds: keys in [w_lo_max, w_hi_min) are visible to every valid row of the wave
     const int wr0 = m0 + wave * 32;
     const int wr1 = min(wr0 + 32, sq_b) - 1;  // last valid row of the wave (may be < wr0 when the wave is empty)
@@ -195,6 +200,13 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
         }
 
         // ---- online softmax (exp2 domain) ---------------------------------------------------------------------
+        if constexpr (kMod) {
+#pragma unroll
+            for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+                for (int j = 0; j < 16; ++j)
+                    s[mbk][j] = rmod.score(s[mbk][j], kb + mbk * 32 + (j >> 2) * 8 + half * 4 + (j & 3));
+        }
         const bool need_mask = (kb < w_lo_max) || (kb + S::BN > w_hi_min);
         float tmax = -INFINITY;
         if (need_mask) {
@@ -212,7 +224,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
 #pragma unroll
             for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
         tmax = pair32_max(tmax);
-        tmax *= a.scale_log2;  // scale > 0: max commutes with the scaling
+        tmax *= scl;  // scale > 0: max commutes with the scaling
         // Lazy rescale: the running reference m_run only moves when some row's maximum outgrows it by more than
         // kLazy (in log2 units).  Softmax is shift invariant, so keeping a stale reference is exact; it bounds the
         // exponentials by 2^kLazy and saves the accumulator rescale on almost every tile.
@@ -232,7 +244,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
         for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
-                const float p = fast_exp2(__builtin_fmaf(s[mbk][j], a.scale_log2, -m_ref));
+                const float p = fast_exp2(__builtin_fmaf(s[mbk][j], scl, -m_ref));
                 s[mbk][j] = p;
                 psum += p;
             }
@@ -285,6 +297,10 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
 {
     const dim3 grid(a.m_tiles, a.hq, a.batch);
     constexpr size_t lds = prefill_lds_bytes<D>();
+    if (a.mod.active()) {
+        if (uniform) return launch_with_lds<prefill_kernel<T, D, true, true>>(grid, dim3(256), lds, st, a);
+        return launch_with_lds<prefill_kernel<T, D, false, true>>(grid, dim3(256), lds, st, a);
+    }
     if (uniform) return launch_with_lds<prefill_kernel<T, D, true>>(grid, dim3(256), lds, st, a);
     return launch_with_lds<prefill_kernel<T, D, false>>(grid, dim3(256), lds, st, a);
 }

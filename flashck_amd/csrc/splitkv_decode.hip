@@ -57,9 +57,10 @@ __device__ __forceinline__ int v_swizzle(int key)
     return ((key & 7) << 1) & (LPR - 1);
 }
 
-template <typename T, int D, int NW, int MB, int HG, bool kUniformPage>
+template <typename T, int D, int NW, int MB, int HG, bool kUniformPage, bool kMod = false>
 __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvArgs a)
 {
+    static_assert(!kMod || HG == 1, "score modifiers are per head: one KV head per workgroup");
     typedef DecodeShape<D, HG> S;
     typedef typename T::vec8 vec8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -131,6 +132,14 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
             lo[mb] = 0;
             hi[mb] = 0;
         }
+    }
+    // bias / ALiBi / soft cap of this lane's rows
+    RowMod<T> rmod[MB];
+    if constexpr (kMod) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            rmod[mb].init(a.mod, b, q_row0, hkv0 * g + row_hl[mb], row_i[mb], sq_b, sk_b, a.mask_type, a.window_left, a.window_right,
+                          a.seqstart_q != nullptr);
     }
     // key range any row of the tile can see (uniform)
     const int i_first = r_tile0 / g;
@@ -314,7 +323,11 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
                     for (int j = 0; j < 4; ++j) {
                         const int key = kb + nb * 16 + kg * 4 + j;
                         const bool vis = key >= lo[mb] && key < hi[mb];
-                        const float v = vis ? s[mb][nb][j] * a.scale_log2 : -INFINITY;
+                        float v;
+                        if constexpr (kMod)
+                            v = vis ? rmod[mb].score(s[mb][nb][j], key) : -INFINITY;
+                        else
+                            v = vis ? s[mb][nb][j] * a.scale_log2 : -INFINITY;
                         x[nb * 4 + j] = v;
                         tmax = fmaxf(tmax, v);
                     }
@@ -511,6 +524,12 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
     const dim3 grid((unsigned)((int64_t)(a.hk / HG) * a.num_splits * a.m_tiles * a.batch));
     const dim3 block(NW * 64);
     constexpr size_t lds = decode_lds_bytes<D, NW, HG>();
+    if constexpr (HG == 1) {
+        if (a.mod.active()) {
+            if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true>>(grid, block, lds, st, a);
+            return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true>>(grid, block, lds, st, a);
+        }
+    }
     if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true>>(grid, block, lds, st, a);
     return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false>>(grid, block, lds, st, a);
 }
@@ -519,7 +538,7 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
 // covers the CUs.
 static bool use_head_pairs(const SplitKvArgs& a, int m_tiles, int num_cu)
 {
-    if (a.hk % 2) return false;
+    if (a.hk % 2 || a.mod.active()) return false;
     return (int64_t)(a.hk / 2) * a.num_splits * m_tiles * a.batch >= num_cu;
 }
 

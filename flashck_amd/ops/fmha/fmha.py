@@ -122,6 +122,53 @@ def _window(window):
     return int(wl), int(wr)
 
 
+def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols):
+    """fck_fmha_attrs for a call, or None when no score modifier is asked for.
+
+    bias (elementwise, BiasEnum ELEMENTWISE_BIAS): q's dtype, last dim contiguous; batch mode [1|B, 1|Hq, sq, >= sk],
+    group mode [1|Hq, total_q, >= max sk]; size-1 dims are shared (the reference's rank 0 / 1 / 2).
+    alibi_slopes (ALIBI): fp32 [Hq] or [B, Hq].  logits_soft_cap > 0: s = cap * tanh(scale * qk / cap).
+    Returns (pointer argument, object to keep alive until the call has been made)."""
+    cap = float(logits_soft_cap)
+    if not (cap >= 0.0) or math.isinf(cap):
+        raise ValueError("logits_soft_cap must be finite and >= 0")
+    if bias is None and alibi_slopes is None and cap == 0.0:
+        return None, None
+    if bias is not None and alibi_slopes is not None:
+        raise ValueError("bias and alibi_slopes are exclusive (one BiasEnum per call)")
+    a = _lib.Attrs()
+    a.size = ctypes.sizeof(_lib.Attrs)
+    a.logits_soft_cap = cap
+    Hq = q.shape[-2]
+    if bias is not None:
+        if not isinstance(bias, torch.Tensor):
+            raise TypeError(f"Expected bias to be a torch.Tensor, got {type(bias)}")
+        if _REQUIRE_GPU_TENSORS and not bias.is_cuda:
+            raise ValueError(f"bias must live on the GPU (got device {bias.device})")
+        if bias.dtype != q.dtype:
+            raise TypeError(f"bias must have q's dtype {q.dtype}, got {bias.dtype}")
+        if bias.dim() != (3 if group else 4) or bias.stride(-1) != 1:
+            raise ValueError(f"bias must be {'[1|Hq, total_q, sk]' if group else '[1|B, 1|Hq, sq, sk]'} with a contiguous last dim, "
+                             f"got shape {tuple(bias.shape)} strides {bias.stride()}")
+        if bias.shape[-3] not in (1, Hq) or (not group and bias.shape[0] not in (1, batch)):
+            raise ValueError(f"bias {tuple(bias.shape)}: head dim must be 1 or {Hq}" + ("" if group else f", batch dim 1 or {batch}"))
+        if bias.shape[-2] != rows or bias.shape[-1] < min_cols:
+            raise ValueError(f"bias {tuple(bias.shape)} must have {rows} rows and at least {min_cols} columns")
+        a.bias_type = 1
+        a.bias = bias.data_ptr()
+        a.bias_row_stride = bias.stride(-2)
+        a.bias_head_stride = bias.stride(-3) if bias.shape[-3] > 1 else 0
+        a.bias_batch_stride = 0 if group or bias.shape[0] == 1 else bias.stride(0)
+    elif alibi_slopes is not None:
+        _check_tensor("alibi_slopes", alibi_slopes, dtype=torch.float32, ndim=(1, 2))
+        if alibi_slopes.shape[-1] != Hq or (alibi_slopes.dim() == 2 and alibi_slopes.shape[0] != batch):
+            raise ValueError(f"alibi_slopes must be [{Hq}] or [{batch}, {Hq}], got {tuple(alibi_slopes.shape)}")
+        a.bias_type = 2
+        a.bias = alibi_slopes.data_ptr()
+        a.bias_batch_stride = Hq if alibi_slopes.dim() == 2 else 0
+    return ctypes.byref(a), (a, bias, alibi_slopes)
+
+
 def num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, num_cu=0) -> int:
     """Split count chosen from the CU count and the KV length."""
     return int(_lib.load().fck_fmha_num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k,
@@ -136,8 +183,10 @@ def splitkv_workspace(shape_batch, q_num_heads, shape_seqlen_q, v_head_dim, num_
 
 
 def fmha_fwd(q, k, v, scale: float = 0.0, mask_type: int = MASK_NONE, window: Tuple[int, int] = (-1, -1),
-             seqlen_k: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Dense attention, batch mode: q [B,sq,Hq,D], k/v [B,sk,Hk,D] -> o [B,sq,Hq,D]."""
+             seqlen_k: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, *, bias=None, alibi_slopes=None,
+             logits_soft_cap: float = 0.0) -> torch.Tensor:
+    """Dense attention, batch mode: q [B,sq,Hq,D], k/v [B,sk,Hk,D] -> o [B,sq,Hq,D].
+    bias / alibi_slopes / logits_soft_cap: see _attrs."""
     _check_tensor("q", q, ndim=4)
     _check_tensor("k", k, dtype=q.dtype, ndim=4)
     _check_tensor("v", v, dtype=q.dtype, ndim=4)
@@ -153,14 +202,22 @@ def fmha_fwd(q, k, v, scale: float = 0.0, mask_type: int = MASK_NONE, window: Tu
     sk, Hk, Dv = k.shape[1], k.shape[2], v.shape[3]
     o = _out("out", out, (B, sq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
-    _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), None, None, _ptr(seqlen_k), B, sq, sk, Hq, Hk, D, Dv,
-          sq, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, False, B, sq, sk)
+    if at is None:
+        _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), None, None, _ptr(seqlen_k), B, sq, sk, Hq, Hk, D, Dv,
+              sq, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    else:
+        _call("fck_fmha_fwd_attrs", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), None, None, _ptr(seqlen_k), B, sq, sk, Hq, Hk, D, Dv,
+              sq, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), at, _stream())
+    del keep
     return o
 
 
 def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scale: float = 0.0,
-                    mask_type: int = MASK_NONE, window=(-1, -1), seqlen_k=None, out=None) -> torch.Tensor:
+                    mask_type: int = MASK_NONE, window=(-1, -1), seqlen_k=None, out=None, *, bias=None, alibi_slopes=None,
+                    logits_soft_cap: float = 0.0) -> torch.Tensor:
     """Dense attention, group mode: q [total_q,Hq,D], k/v [total_k,Hk,D] packed by cu_seqlens.
+    bias / alibi_slopes / logits_soft_cap: see _attrs.
 
     seqlen_k (int32 [B], optional): logical key counts when the packed K/V slots hold padding behind the keys."""
     _check_tensor("q", q, ndim=3)
@@ -179,15 +236,23 @@ def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scal
     Hk, Dv = k.shape[1], v.shape[2]
     o = _out("out", out, (tq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
-    _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), _ptr(seqlen_k), B, tq,
-          k.shape[0], Hq, Hk, D, Dv, max_seqlen_q, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1)
+    if at is None:
+        _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), _ptr(seqlen_k), B, tq,
+              k.shape[0], Hq, Hk, D, Dv, max_seqlen_q, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    else:
+        _call("fck_fmha_fwd_attrs", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), _ptr(seqlen_k),
+              B, tq, k.shape[0], Hq, Hk, D, Dv, max_seqlen_q, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), at, _stream())
+    del keep
     return o
 
 
 def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=None, cache_batch_idx=None,
                      cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q: int = 0, scale: float = 0.0,
-                     mask_type: int = MASK_NONE, window=(-1, -1), o_acc=None, lse_acc=None):
+                     mask_type: int = MASK_NONE, window=(-1, -1), o_acc=None, lse_acc=None, bias=None, alibi_slopes=None,
+                     logits_soft_cap: float = 0.0):
     """Split-KV forward: returns the per-split partials (o_acc, lse_acc), to be merged by fmha_fwd_splitkv_combine.
+    bias / alibi_slopes / logits_soft_cap: see _attrs.
 
     k/v are a paged cache when block_table is given, packed when cu_seqlens_k is given, else [B*, sk, Hk, D].
     """
@@ -232,9 +297,16 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
         _check_shape("o_acc", o_acc, (bs, Hq, int(num_splits), sq, Dv), q)
         _check_shape("lse_acc", lse_acc, (bs, Hq, int(num_splits), sq), q)
     wl, wr = _window(window)
-    _call("fck_fmha_fwd_splitkv", _ptr(q), _ptr(k), _ptr(v), None, _ptr(lse_acc), _ptr(o_acc), _ptr(cu_seqlens_q),
-          _ptr(cu_seqlens_k), _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv,
-          max_seqlen_q, int(num_splits), max_blocks, page, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, sq, 1 if (group or block_table is not None) else sk)
+    if at is None:
+        _call("fck_fmha_fwd_splitkv", _ptr(q), _ptr(k), _ptr(v), None, _ptr(lse_acc), _ptr(o_acc), _ptr(cu_seqlens_q),
+              _ptr(cu_seqlens_k), _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv,
+              max_seqlen_q, int(num_splits), max_blocks, page, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    else:
+        _call("fck_fmha_fwd_splitkv_attrs", _ptr(q), _ptr(k), _ptr(v), None, _ptr(lse_acc), _ptr(o_acc), _ptr(cu_seqlens_q),
+              _ptr(cu_seqlens_k), _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv,
+              max_seqlen_q, int(num_splits), max_blocks, page, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), at, _stream())
+    del keep
     return o_acc, lse_acc
 
 
@@ -386,7 +458,7 @@ def fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, *, cu_seqlens_k
 
 def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_indices, kv_last_page_lens=None, *,
                        max_seqlen_q: int, scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0),
-                       out=None) -> torch.Tensor:
+                       out=None, bias=None, alibi_slopes=None, logits_soft_cap: float = 0.0) -> torch.Tensor:
     """Varlen prefill over a page list: q [total_q,Hq,D]; sequence b owns pages
     kv_page_indices[kv_indptr[b]:kv_indptr[b+1]] of the cache [num_pages, page_size, Hk, D]."""
     _check_tensor("q", q, ndim=3)
@@ -405,14 +477,22 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
     num_pages, page, Hk, Dv = v_cache.shape
     o = _out("out", out, (tq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
-    _call("fck_fmha_batch_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
-          _ptr(kv_page_indices), _ptr(kv_last_page_lens), num_pages, page, B, Hq, Hk, D, Dv, max_seqlen_q,
-          _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1)
+    if at is None:
+        _call("fck_fmha_batch_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
+              _ptr(kv_page_indices), _ptr(kv_last_page_lens), num_pages, page, B, Hq, Hk, D, Dv, max_seqlen_q,
+              _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
+    else:
+        _call("fck_fmha_batch_prefill_attrs", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
+              _ptr(kv_page_indices), _ptr(kv_last_page_lens), num_pages, page, B, Hq, Hk, D, Dv, max_seqlen_q,
+              _scale(scale, D), wl, wr, mask_type, _dtype_id(q), at, _stream())
+    del keep
     return o
 
 
 def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q=None, max_seqlen_q: int = 0,
-                     scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0), out=None) -> torch.Tensor:
+                     scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0), out=None, bias=None,
+                     alibi_slopes=None, logits_soft_cap: float = 0.0) -> torch.Tensor:
     """Prefill over a block table (no splits): q [B,sq,Hq,D] or packed [total_q,Hq,D]."""
     group = cu_seqlens_q is not None
     _check_tensor("q", q, ndim=3 if group else 4)
@@ -434,9 +514,16 @@ def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q
         raise ValueError("group mode needs max_seqlen_q")
     o = _out("out", out, (*q.shape[:-1], Dv), q.dtype, q)
     wl, wr = _window(window)
-    _call("fck_fmha_fwd_pagedkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
-          _ptr(block_table), block_table.shape[1], page, B, sq, Hq, Hk, D, Dv, max_seqlen_q or sq, _scale(scale, D), wl, wr,
-          mask_type, _dtype_id(q), _stream())
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, q.shape[0] if group else sq, 1)
+    if at is None:
+        _call("fck_fmha_fwd_pagedkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
+              _ptr(block_table), block_table.shape[1], page, B, sq, Hq, Hk, D, Dv, max_seqlen_q or sq, _scale(scale, D), wl, wr,
+              mask_type, _dtype_id(q), _stream())
+    else:
+        _call("fck_fmha_fwd_pagedkv_attrs", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
+              _ptr(block_table), block_table.shape[1], page, B, sq, Hq, Hk, D, Dv, max_seqlen_q or sq, _scale(scale, D), wl, wr,
+              mask_type, _dtype_id(q), at, _stream())
+    del keep
     return o
 
 

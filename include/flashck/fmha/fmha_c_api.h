@@ -51,6 +51,39 @@ extern "C" {
 #define FCK_ROPE_INTERLEAVED 1
 #define FCK_ROPE_HALF_ROTATED 2
 
+/* BiasEnum, core/profiling/attention/fmha_library.h:121-126 */
+#define FCK_BIAS_NONE 0
+#define FCK_BIAS_ELEMENTWISE 1
+#define FCK_BIAS_ALIBI 2
+
+/*
+ * What FlashCK fixes per generated kernel instance and this library takes per call: the bias kind and its rank
+ * (core/profiling/attention/fmha_library.h:150-165, stride plumbing
+ * core/module/kernels/attention_kernels/fmha_fwd_split_kv/fmha_fwd_split_kv_jinja.h:359-385) and the logits soft cap
+ * (core/profiling/attention/fmha_fwd_split_kv/fmha_fwd_split_kv_problem.h:81).  Passed to the *_attrs entry points;
+ * a NULL pointer (or the entry point without the suffix) means none of them.
+ *
+ * Scores: x = scale * q.k;  x = cap * tanh(x / cap) when logits_soft_cap > 0;  x += bias;  then the mask.
+ *   ELEMENTWISE_BIAS  T elements; (b, h, i, j) at bias[b * bias_batch_stride + h * bias_head_stride + i * bias_row_stride + j].
+ *                     The reference's rank 0 (1*1*s*s) is head and batch stride 0, rank 1 (1*h*s*s) batch stride 0,
+ *                     rank 2 (b*h*s*s) neither.  Group mode: i counts packed query rows (seqstart_q[b] + local row)
+ *                     and bias_batch_stride is not used.
+ *   ALIBI             fp32 slopes; (b, h) at bias[b * bias_batch_stride + h]: rank 0 (1*h) is batch stride 0, rank 1 (b*h)
+ *                     is q_num_heads.  The term added is slope * j for a causal window (window_left < 0, window_right == 0,
+ *                     mask_type != NONE), else -slope * |i - j| (top-left) or -slope * |i + sk - sq - j| (bottom-right,
+ *                     and no mask).
+ */
+typedef struct fck_fmha_attrs {
+    uint32_t size;             /* sizeof(fck_fmha_attrs) */
+    int32_t bias_type;         /* FCK_BIAS_* */
+    const void* bias;          /* used by the entry points without a bias argument (or when that argument is NULL) */
+    int64_t bias_batch_stride; /* elements */
+    int64_t bias_head_stride;
+    int64_t bias_row_stride;
+    float logits_soft_cap;     /* > 0: on; 0: off */
+    uint32_t reserved;         /* 0 */
+} fck_fmha_attrs;
+
 #define FCK_OK 0
 #define FCK_ERR_INVALID_ARGUMENT (-1) /* null pointer, non-positive size, Hq % Hk != 0 ... */
 #define FCK_ERR_UNSUPPORTED (-2)      /* dtype / head_dim / feature this build has no kernel for */
@@ -78,6 +111,14 @@ FCK_EXPORT int fck_fmha_fwd(const void* q, const void* k, const void* v, const v
                             int64_t kv_num_heads, int64_t qk_head_dim, int64_t v_head_dim, int64_t q_max_seq_len,
                             float scale, int64_t window_left, int64_t window_right, uint32_t mask_type,
                             int32_t dtype, void* stream);
+/* The same with bias / ALiBi / soft cap (`attrs` may be NULL): the instances FlashCK generates for
+ * bias_str != "no" (fmha_fwd/fmha_fwd_jinja.h:124-147, BiasEnum fmha_library.h:121-126). */
+FCK_EXPORT int fck_fmha_fwd_attrs(const void* q, const void* k, const void* v, const void* bias, void* o,
+                                  const int32_t* seqstart_q, const int32_t* seqstart_k, const int32_t* seqlen_k_ptr,
+                                  int64_t batch, int64_t seqlen_q, int64_t seqlen_k, int64_t q_num_heads,
+                                  int64_t kv_num_heads, int64_t qk_head_dim, int64_t v_head_dim, int64_t q_max_seq_len,
+                                  float scale, int64_t window_left, int64_t window_right, uint32_t mask_type,
+                                  int32_t dtype, const fck_fmha_attrs* attrs, void* stream);
 
 /*
  * Split-KV forward: per split s of num_splits, attention over keys [s*ceil(Lk/ns), min(Lk,(s+1)*ceil(Lk/ns)))
@@ -96,6 +137,17 @@ FCK_EXPORT int fck_fmha_fwd_splitkv(const void* q, const void* k, const void* v,
                                     int64_t max_num_page_blocks, int64_t page_block_size, float scale,
                                     int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype,
                                     void* stream);
+/* The same with bias / ALiBi / soft cap (`attrs` may be NULL): the instances FlashCK generates for
+ * bias_str != "no" or has_logits_soft_cap (fmha_fwd_split_kv_jinja.h:359-385, fmha_fwd_split_kv_problem.h:81). */
+FCK_EXPORT int fck_fmha_fwd_splitkv_attrs(const void* q, const void* k, const void* v, const void* bias, void* lse_acc,
+                                          void* o_acc, const int32_t* seqstart_q, const int32_t* seqstart_k,
+                                          const int32_t* seqlen_k_ptr, const int32_t* block_table,
+                                          const int32_t* cache_batch_idx, int64_t batch, int64_t seqlen_q,
+                                          int64_t seqlen_k, int64_t q_num_heads, int64_t kv_num_heads,
+                                          int64_t qk_head_dim, int64_t v_head_dim, int64_t q_max_seq_len,
+                                          int64_t num_splits, int64_t max_num_page_blocks, int64_t page_block_size,
+                                          float scale, int64_t window_left, int64_t window_right, uint32_t mask_type,
+                                          int32_t dtype, const fck_fmha_attrs* attrs, void* stream);
 
 /*
  * Split-KV forward and LSE combine in ONE launch that allocates nothing: fck_fmha_fwd_splitkv with `o` in place of
@@ -171,6 +223,16 @@ FCK_EXPORT int fck_fmha_batch_prefill(const void* q, const void* k_cache, const 
                                       int64_t q_num_heads, int64_t kv_num_heads, int64_t qk_head_dim,
                                       int64_t v_head_dim, int64_t q_max_seq_len, float scale, int64_t window_left,
                                       int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream);
+/* The same with bias / ALiBi / soft cap; the bias pointer travels in `attrs` (BiasEnum and has_logits_soft_cap of
+ * core/profiling/attention/fmha_fwd_batch_prefill/fmha_fwd_batch_prefill_problem.h:35-100). */
+FCK_EXPORT int fck_fmha_batch_prefill_attrs(const void* q, const void* k_cache, const void* v_cache, void* o,
+                                            const int32_t* seqstart_q, const int32_t* kv_indptr,
+                                            const int32_t* kv_page_indices, const int32_t* kv_last_page_lens,
+                                            int64_t num_total_pages, int64_t page_block_size, int64_t batch,
+                                            int64_t q_num_heads, int64_t kv_num_heads, int64_t qk_head_dim,
+                                            int64_t v_head_dim, int64_t q_max_seq_len, float scale,
+                                            int64_t window_left, int64_t window_right, uint32_t mask_type,
+                                            int32_t dtype, const fck_fmha_attrs* attrs, void* stream);
 
 /*
  * Prefill over a vLLM-style block table (no splits).  FlashCK's problem definition:
@@ -184,6 +246,16 @@ FCK_EXPORT int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const vo
                                     int64_t kv_num_heads, int64_t qk_head_dim, int64_t v_head_dim,
                                     int64_t q_max_seq_len, float scale, int64_t window_left, int64_t window_right,
                                     uint32_t mask_type, int32_t dtype, void* stream);
+/* The same with bias / ALiBi / soft cap; the bias pointer travels in `attrs`
+ * (core/profiling/attention/fmha_fwd_paged_kv_prefill/fmha_fwd_paged_kv_prefill_problem.h:35-97). */
+FCK_EXPORT int fck_fmha_fwd_pagedkv_attrs(const void* q, const void* k_cache, const void* v_cache, void* o,
+                                          const int32_t* seqstart_q, const int32_t* seqlen_k_ptr,
+                                          const int32_t* block_table, int64_t batch_stride_block_table,
+                                          int64_t page_block_size, int64_t batch, int64_t seqlen_q,
+                                          int64_t q_num_heads, int64_t kv_num_heads, int64_t qk_head_dim,
+                                          int64_t v_head_dim, int64_t q_max_seq_len, float scale,
+                                          int64_t window_left, int64_t window_right, uint32_t mask_type,
+                                          int32_t dtype, const fck_fmha_attrs* attrs, void* stream);
 
 /*
  * Split count from the CU count and the KV length.  FlashCK's command line promises "0 = heuristic"

@@ -215,7 +215,7 @@ typedef struct {
 } scratch_t;
 
 /* Returns lse through *lse_out; writes normalised fp32 output (P rounded to the data type first) into of[]. */
-static void attend_row(const fck_orc_problem* p, const void* q, const void* k, const void* v, int64_t qrow, int h,
+static void attend_row(const fck_orc_problem* p, const void* q, const void* k, const void* v, int b, int64_t qrow, int h,
                        const int64_t* rows, int k0, int k1, int i, int sq_b, int sk_b, scratch_t* sc, float* lse_out)
 {
     const int d = p->d, dv = p->dv, hk = p->hk, dt = p->dtype;
@@ -224,12 +224,42 @@ static void attend_row(const fck_orc_problem* p, const void* q, const void* k, c
     mask_coords(p->mask_type, p->window_left, p->window_right, sq_b, sk_b, &y, &x);
     for (int t = 0; t < d; ++t) sc->qf[t] = ld(q, (qrow * p->hq + h) * d + t, dt);
 
+    /* bias row of (b, h, i) / ALiBi slope of (b, h) */
+    int64_t bias_row = 0;
+    float slope = 0.f;
+    int alibi_mode = 2;
+    if (p->bias_type == 1) {
+        bias_row = (int64_t)h * p->bias_head_stride +
+                   (p->seqstart_q ? qrow * p->bias_row_stride : (int64_t)b * p->bias_batch_stride + (int64_t)i * p->bias_row_stride);
+    } else if (p->bias_type == 2) {
+        slope = ((const float*)p->bias)[(int64_t)b * p->bias_batch_stride + h];
+        /* make_alibi_from_lr_mask: a causal window is VERTICAL, else the mask enum names the diagonal; no mask:
+           FROM_BOTTOM_RIGHT */
+        if (p->mask_type == 0)
+            alibi_mode = 2;
+        else if (p->window_left < 0 && p->window_right == 0)
+            alibi_mode = 0;
+        else
+            alibi_mode = p->mask_type == 1 ? 1 : 2;
+    }
+
     float vmax = -INFINITY;
     for (int j = k0; j < k1; ++j) {
         float acc = 0.f;
         const int64_t base = (rows[j] * hk + hkv) * d;
         for (int t = 0; t < d; ++t) acc += sc->qf[t] * ld(k, base + t, dt);
         float sv = acc * p->scale;
+        if (p->logits_soft_cap > 0.f) sv = p->logits_soft_cap * tanhf(sv / p->logits_soft_cap);
+        if (p->bias_type == 1) {
+            sv += ld(p->bias, bias_row + j, dt);
+        } else if (p->bias_type == 2) {
+            /* Alibi::update (row major): VERTICAL adds slope * col; the two diagonal modes add -slope * |zero - col| with
+               zero = row (top left) or row + sk - sq (bottom right: shift_right_down - shift_left_up = sk - sq) */
+            if (alibi_mode == 0)
+                sv += slope * (float)j;
+            else
+                sv += -slope * (float)labs((long)(alibi_mode == 1 ? i : i + sk_b - sq_b) - (long)j);
+        }
         if (!visible_yx(p->mask_type, y, x, sk_b, i, j)) sv = -INFINITY;
         sc->s[j - k0] = sv;
         vmax = vmax < sv ? sv : vmax;
@@ -294,7 +324,7 @@ int fck_orc_fmha_fwd(const fck_orc_problem* p, const void* q, const void* k, con
             for (int64_t t = 0; t < ntask; ++t) {
                 const int h = (int)(t / sq_b), i = (int)(t % sq_b);
                 float l;
-                attend_row(p, q, k, v, row0 + i, h, rows, 0, sk_b, i, sq_b, sk_b, &sc, &l);
+                attend_row(p, q, k, v, b, row0 + i, h, rows, 0, sk_b, i, sq_b, sk_b, &sc, &l);
                 uint16_t* orow = (uint16_t*)o + ((row0 + i) * p->hq + h) * p->dv;
                 for (int c = 0; c < p->dv; ++c) orow[c] = cvt(sc.of[c], p->dtype);
                 if (lse) {
@@ -353,7 +383,7 @@ int fck_orc_fmha_splitkv(const fck_orc_problem* p, const void* q, const void* k,
                 if (k1 > sk_b) k1 = sk_b;
                 if (k0 > k1) k0 = k1;
                 float l;
-                attend_row(p, q, k, v, row0 + i, h, rows, k0, k1, i, sq_b, sk_b, &sc, &l);
+                attend_row(p, q, k, v, b, row0 + i, h, rows, k0, k1, i, sq_b, sk_b, &sc, &l);
                 const int64_t w = ((wb * p->hq + h) * num_splits + s) * Sq + wrow0 + i;
                 lse_acc[w] = l;
                 for (int c = 0; c < p->dv; ++c) o_acc[w * p->dv + c] = isinf(l) ? 0.f : sc.of[c];

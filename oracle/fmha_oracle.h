@@ -58,6 +58,18 @@ typedef struct {
     float scale;
     int32_t mask_type;
     int64_t window_left, window_right;
+    /* Score modifiers, applied in this order before the mask (ck_tile/ops/fmha/pipeline/
+       block_fmha_pipeline_qr_ks_vs.hpp:391-449): soft cap, then bias.
+       BiasEnum: core/profiling/attention/fmha_library.h:121-126 (rank rule :150-165).
+         1 elementwise: data dtype, (b, h, i, j) at bias[b*bias_batch_stride + h*bias_head_stride + i*bias_row_stride + j];
+           group mode: i counts packed query rows, no batch stride (ck_tile/ops/fmha/kernel/fmha_fwd_splitkv_kernel.hpp:608-688)
+         2 ALiBi: fp32 slopes, (b, h) at bias[b*bias_batch_stride + h]; term and mode:
+           ck_tile/ops/fmha/block/block_position_encoding.hpp:19-121,138-152, ck_tile/ops/fmha/kernel/fmha_fwd_kernel.hpp:1482-1507
+       logits_soft_cap > 0: s = cap * tanh(scale * qk / cap), ck_tile/ops/fmha/block/variants.hpp:208-209 */
+    int32_t bias_type;
+    const void* bias;
+    int64_t bias_batch_stride, bias_head_stride, bias_row_stride;
+    float logits_soft_cap;
 } fck_orc_problem;
 
 /* 1 when key j is visible to query i. */

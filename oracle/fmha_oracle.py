@@ -41,6 +41,10 @@ class _Problem(ctypes.Structure):
         ("scale", ctypes.c_float),
         ("mask_type", ctypes.c_int32),
         ("window_left", ctypes.c_int64), ("window_right", ctypes.c_int64),
+        ("bias_type", ctypes.c_int32),
+        ("bias", ctypes.c_void_p),
+        ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64),
+        ("logits_soft_cap", ctypes.c_float),
     ]
 
 
@@ -98,7 +102,9 @@ def _i32(t):
 
 def _problem(q, k, v, *, seqstart_q=None, seqstart_k=None, seqlen_k=None, block_table=None, page_size=0,
              kv_indptr=None, kv_page_indices=None, kv_last_page_lens=None, cache_batch_idx=None, scale=None,
-             mask_type=NO_MASK, window=(-1, -1), batch=None):
+             mask_type=NO_MASK, window=(-1, -1), batch=None, bias=None, alibi_slopes=None, logits_soft_cap=0.0):
+    """bias: data dtype, [1|B, 1|Hq, sq, sk] (batch mode) or [1|Hq, total_q, max_sk] (group mode), last dim contiguous;
+    alibi_slopes: fp32 [Hq] or [B, Hq]; logits_soft_cap > 0: s = cap * tanh(scale * qk / cap)."""
     p = _Problem()
     p.dtype = dtype_id(q.dtype)
     p.hq, p.d = q.shape[-2], q.shape[-1]
@@ -135,6 +141,24 @@ def _problem(q, k, v, *, seqstart_q=None, seqstart_k=None, seqlen_k=None, block_
     p.scale = float(scale if scale is not None else q.shape[-1] ** -0.5)
     p.mask_type = int(mask_type)
     p.window_left, p.window_right = int(window[0]), int(window[1])
+    p.logits_soft_cap = float(logits_soft_cap)
+    assert bias is None or alibi_slopes is None, "one bias kind at a time"
+    if bias is not None:
+        assert bias.dtype == q.dtype and bias.device.type == "cpu" and bias.stride(-1) == 1
+        group = seqstart_q is not None
+        assert bias.dim() == (3 if group else 4)
+        p.bias_type = 1
+        p.bias = bias.data_ptr()
+        p.bias_row_stride = bias.stride(-2)
+        p.bias_head_stride = bias.stride(-3) if bias.shape[-3] > 1 else 0
+        p.bias_batch_stride = 0 if group or bias.shape[0] == 1 else bias.stride(0)
+        p._keep = bias
+    elif alibi_slopes is not None:
+        assert alibi_slopes.dtype == torch.float32 and alibi_slopes.is_contiguous() and alibi_slopes.shape[-1] == p.hq
+        p.bias_type = 2
+        p.bias = alibi_slopes.data_ptr()
+        p.bias_batch_stride = p.hq if alibi_slopes.dim() == 2 else 0
+        p._keep = alibi_slopes
     return p
 
 
