@@ -60,6 +60,7 @@ def parse():
     ap.add_argument("--kv-len", type=int, default=32768, help="KV length of the split-KV workload (study runs only)")
     ap.add_argument("--no-shuffle", action="store_true", help="identity page order (study runs only)")
     ap.add_argument("--num-splits", type=int, default=8, help="split count of the split-KV workload (study runs only)")
+    ap.add_argument("--kv-fp8", action="store_true", help="split-KV workload with the cache stored as fp8 (e4m3, static scales)")
     ap.add_argument("--decode-path", default="two-launch", choices=["two-launch", "fused"],
                     help="two-launch: split-KV + combine kernels with a caller-owned workspace; fused: one launch "
                          "(--num-splits 0 lets the library choose the key ranges)")
@@ -125,6 +126,14 @@ def bench_decode(args, torch, fmha, gen, which):
     dev = "cuda"
     q = w["q"].to(dev)
     bt, sl = w["block_table"].to(dev), w["seqlen_k"].to(dev)
+    kv_fp8 = getattr(args, "kv_fp8", False)
+    scales = {}
+    if kv_fp8:
+        # unit-variance data: a static scale of 1/16 keeps it well inside the e4m3 range (+-448)
+        scales = dict(k_descale=0.0625, v_descale=0.0625)
+        w["k_cache"] = (w["k_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
+        w["v_cache"] = (w["v_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
+        name += " [K/V cache fp8 e4m3]"
     pools = [(w["k_cache"].to(dev), w["v_cache"].to(dev))]
     for _ in range(args.copies - 1):
         pools.append((pools[0][0].clone(), pools[0][1].clone()))
@@ -140,7 +149,7 @@ def bench_decode(args, torch, fmha, gen, which):
         if fused:
             fmha.fmha_fwd_splitkv_fused(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], out=o)
         else:
-            fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc)
+            fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc, **scales)
         if ev is not None:
             ev[1].record()
         if not fused:
@@ -148,7 +157,7 @@ def bench_decode(args, torch, fmha, gen, which):
 
     wall, kern_ms = time_steps(step, args.steps, args.warmup, torch, kernel_events="region" if fused else True)
     kernel = _lib.load().fck_fmha_last_kernel().decode()  # the combine launch does not change it
-    nbytes = gen.decode_bytes(w["lens"], [1] * B, Hq, Hk, D, D, 128)
+    nbytes = gen.decode_bytes(w["lens"], [1] * B, Hq, Hk, D, D, 128, kv_elem=1 if kv_fp8 else None)
     flops = gen.decode_flops(w["lens"], [1] * B, Hq, D, D)
     ms = wall / args.steps * 1e3
     res = dict(name=name, ms_per_step=ms, bytes=nbytes, flops=flops, gbs=nbytes / (ms * 1e-3) / 1e9,
@@ -298,9 +307,9 @@ def main():
                         mfma_util_pct=100 * r5["tflops"] / MFMA_BF16_PEAK_TFLOPS, flops=r5["flops"], kernel_ms=r5["kernel_ms"],
                         kernel=r5["kernel"])
 
-        def splitkv_variant(path, ns):
+        def splitkv_variant(path, ns, kv_fp8=False):
             a2 = argparse.Namespace(**vars(args))
-            a2.steps, a2.warmup, a2.decode_path, a2.num_splits = max(20, args.steps // 2), 10, path, ns
+            a2.steps, a2.warmup, a2.decode_path, a2.num_splits, a2.kv_fp8 = max(20, args.steps // 2), 10, path, ns, kv_fp8
             r3 = bench_decode(a2, torch, fmha, gen, "splitkv")
             return dict(workload=r3["name"], us_per_call=r3["ms_per_step"] * 1e3, gbs=r3["gbs"],
                         pct_of_hbm_peak=100 * r3["gbs"] / HBM_PEAK_GBS, kernel_us=r3["kernel_ms"] * 1e3, num_splits=r3["num_splits"])
@@ -309,6 +318,7 @@ def main():
         ns_lib = fmha.num_splits_heuristic(4, 64, 8, 1, args.kv_len, 128)
         secondary("splitkv_library_splits", lambda: splitkv_variant("two-launch", ns_lib))
         secondary("splitkv_fused", lambda: splitkv_variant("fused", 0))
+        secondary("splitkv_fp8_cache", lambda: splitkv_variant("two-launch", ns_lib, kv_fp8=True))
         secondary("paged_decode", paged)
         secondary("appendkv", append)
         for d in (128, 256):

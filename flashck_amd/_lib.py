@@ -16,7 +16,8 @@ class Attrs(ctypes.Structure):
     """fck_fmha_attrs of the header."""
     _fields_ = [("size", ctypes.c_uint32), ("bias_type", ctypes.c_int32), ("bias", ctypes.c_void_p),
                 ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64),
-                ("logits_soft_cap", ctypes.c_float), ("reserved", ctypes.c_uint32)]
+                ("logits_soft_cap", ctypes.c_float), ("kv_dtype", ctypes.c_int32), ("k_descale", ctypes.c_float),
+                ("v_descale", ctypes.c_float)]
 
 
 _ap = ctypes.POINTER(Attrs)

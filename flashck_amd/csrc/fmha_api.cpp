@@ -39,6 +39,13 @@ int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, i
 }
 
 // Bias / ALiBi / soft cap of a call: `bias` is the positional pointer of the entry points that have one (else null).
+int no_kv_dtype(const fck_fmha_attrs* at)
+{
+    if (at && at->size == sizeof(fck_fmha_attrs) && at->kv_dtype != 0)
+        return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: a K/V cache type other than q's is read by the split-KV entry point only", at->kv_dtype);
+    return FCK_OK;
+}
+
 int fill_mod(fck::ScoreMod& m, const void* bias, const fck_fmha_attrs* at, float scale, uint32_t mask_type, int64_t hq)
 {
     m = fck::ScoreMod{};
@@ -191,6 +198,19 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
+    a.v_descale = 1.f;
+    if (attrs && attrs->kv_dtype != 0) {
+        // fp8 K/V with static per-tensor scales: the K scale multiplies every score, the V scale the output
+        if (attrs->kv_dtype != FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: only 0 (same as q) and FLOAT8 (1)", attrs->kv_dtype);
+        const float kd = attrs->k_descale == 0.f ? 1.f : attrs->k_descale, vd = attrs->v_descale == 0.f ? 1.f : attrs->v_descale;
+        if (!(kd > 0.f) || !std::isfinite(kd) || !(vd > 0.f) || !std::isfinite(vd))
+            return fail(FCK_ERR_INVALID_ARGUMENT, "k_descale and v_descale must be positive and finite (0: 1)");
+        if (!aligned16(k) || !aligned16(v)) return fail(FCK_ERR_INVALID_ARGUMENT, "k and v must be 16-byte aligned");
+        a.kv8 = 1;
+        a.scale_log2 *= kd;
+        a.mod.scale *= kd;
+        a.v_descale = vd;
+    }
 
     uniform = true;
     fck::KvAddr& kv = a.kv;
@@ -252,8 +272,12 @@ int fck_fmha_fwd_splitkv_attrs(const void* q, const void* k, const void* v, cons
     if (!aligned16(o_acc)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_acc must be 16-byte aligned");
     a.o_acc = static_cast<float*>(o_acc);
     a.lse_acc = static_cast<float*>(lse_acc);
-    g_kernel = a.mod.active() ? (uniform ? "splitkv_decode_kernel<uniform_page,score_mod>" : "splitkv_decode_kernel<row_lookup,score_mod>")
-                              : (uniform ? "splitkv_decode_kernel<uniform_page>" : "splitkv_decode_kernel<row_lookup>");
+    static const char* const names[8] = {
+        "splitkv_decode_kernel<row_lookup>",         "splitkv_decode_kernel<uniform_page>",
+        "splitkv_decode_kernel<row_lookup,score_mod>", "splitkv_decode_kernel<uniform_page,score_mod>",
+        "splitkv_decode_kernel<row_lookup,kv_fp8>",  "splitkv_decode_kernel<uniform_page,kv_fp8>",
+        "splitkv_decode_kernel<row_lookup,kv_fp8,score_mod>", "splitkv_decode_kernel<uniform_page,kv_fp8,score_mod>"};
+    g_kernel = names[(a.kv8 ? 4 : 0) + (a.mod.active() ? 2 : 0) + (uniform ? 1 : 0)];
     return launch_status(fck::launch_splitkv_decode(a, (int)d, dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
                          "FmhaFwdSplitKV launch");
 }
@@ -450,6 +474,7 @@ int fck_fmha_fwd_attrs(const void* q, const void* k, const void* v, const void* 
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
+    if (int rc = no_kv_dtype(attrs)) return rc;
     a.kv.page_shift = -1;
     a.kv.seqlen_k_ptr = seqlen_k_ptr;  // group mode: logical key counts of padded packed sequences
     if (seqstart_q) {
@@ -503,6 +528,7 @@ int fck_fmha_batch_prefill_attrs(const void* q, const void* k_cache, const void*
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
+    if (int rc = no_kv_dtype(attrs)) return rc;
     a.kv.mode = 3;
     a.kv.kv_indptr = kv_indptr;
     a.kv.kv_page_indices = kv_page_indices;
@@ -555,6 +581,7 @@ int fck_fmha_fwd_pagedkv_attrs(const void* q, const void* k_cache, const void* v
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
+    if (int rc = no_kv_dtype(attrs)) return rc;
     a.kv.mode = 2;
     a.kv.block_table = block_table;
     a.kv.block_table_stride = (int32_t)batch_stride_block_table;

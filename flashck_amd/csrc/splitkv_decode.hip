@@ -23,6 +23,8 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
+#include <type_traits>
+
 namespace fck {
 
 template <int D, int HG>
@@ -57,7 +59,9 @@ __device__ __forceinline__ int v_swizzle(int key)
     return ((key & 7) << 1) & (LPR - 1);
 }
 
-template <typename T, int D, int NW, int MB, int HG, bool kUniformPage, bool kMod = false>
+// kKv8: K and V are stored as fp8 (e4m3, one byte per element) and widened to T on their way into LDS; everything after
+// the staging tile is the 16-bit path.  A lane then loads 8 bytes where the 16-bit path loads 16.
+template <typename T, int D, int NW, int MB, int HG, bool kUniformPage, bool kMod = false, bool kKv8 = false>
 __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvArgs a)
 {
     static_assert(!kMod || HG == 1, "score modifiers are per head: one KV head per workgroup");
@@ -185,8 +189,27 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
             for (int db = 0; db < S::DB; ++db) oacc[hl][mb][db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
         }
 
-    const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k);
-    const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v);
+    typedef typename std::conditional<kKv8, uint8_t, uint16_t>::type kv_elem;
+    const kv_elem* kp = reinterpret_cast<const kv_elem*>(a.k);
+    const kv_elem* vp = reinterpret_cast<const kv_elem*>(a.v);
+    // one lane's piece of a K/V row: 8 elements, as they come from memory and as they go to LDS
+    auto fetch = [](const kv_elem* p) -> u32x4_t {
+        if constexpr (kKv8) {
+            const u32x2_t v = *reinterpret_cast<const u32x2_t*>(p);
+            return u32x4_t{v[0], v[1], 0u, 0u};
+        } else {
+            return ldg16(p);
+        }
+    };
+    auto staged = [](u32x4_t v) -> u32x4_t {
+        if constexpr (kKv8) {
+            const f32x2_t a0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[0], false), a1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[0], true);
+            const f32x2_t a2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[1], false), a3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[1], true);
+            return u32x4_t{T::pack2(a0[0], a0[1]), T::pack2(a1[0], a1[1]), T::pack2(a2[0], a2[1]), T::pack2(a3[0], a3[1])};
+        } else {
+            return v;
+        }
+    };
     const int64_t krow_stride = (int64_t)a.hk * D;
     const int last_key = sk_b - 1;
 
@@ -262,28 +285,28 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
     };
     auto load_tile = [&](int c, int64_t row0, Frag& f) {
 #pragma unroll
-        for (int u = 0; u < S::VN; ++u) f.a[u] = ldg16(kp + src_off(c, u, row0));
+        for (int u = 0; u < S::VN; ++u) f.a[u] = fetch(kp + src_off(c, u, row0));
 #pragma unroll
-        for (int u = 0; u < S::VN; ++u) f.a[S::VN + u] = ldg16(vp + src_off(c, u, row0));
+        for (int u = 0; u < S::VN; ++u) f.a[S::VN + u] = fetch(vp + src_off(c, u, row0));
     };
     auto store_tile = [&](const Frag& f) {
 #pragma unroll
-        for (int u = 0; u < S::VN; ++u) *(u32x4_t FCK_LDS*)(kstage + kw_off[u]) = f.a[u];
+        for (int u = 0; u < S::VN; ++u) *(u32x4_t FCK_LDS*)(kstage + kw_off[u]) = staged(f.a[u]);
 #pragma unroll
-        for (int u = 0; u < S::VN; ++u) *(u32x4_t FCK_LDS*)(vstage + vw_off[u]) = f.a[S::VN + u];
+        for (int u = 0; u < S::VN; ++u) *(u32x4_t FCK_LDS*)(vstage + vw_off[u]) = staged(f.a[S::VN + u]);
     };
     // write the tile held in f to LDS and request tile c_next into the same registers, one register at a time
     auto refill_tile = [&](int c_next, int64_t row0, Frag& f) {
 #pragma unroll
         for (int u = 0; u < S::VN; ++u) {
-            *(u32x4_t FCK_LDS*)(kstage + kw_off[u]) = f.a[u];
-            f.a[u] = ldg16(kp + src_off(c_next, u, row0));
+            *(u32x4_t FCK_LDS*)(kstage + kw_off[u]) = staged(f.a[u]);
+            f.a[u] = fetch(kp + src_off(c_next, u, row0));
             __builtin_amdgcn_sched_barrier(0);  // keep the store / load pairs interleaved in this order
         }
 #pragma unroll
         for (int u = 0; u < S::VN; ++u) {
-            *(u32x4_t FCK_LDS*)(vstage + vw_off[u]) = f.a[S::VN + u];
-            f.a[S::VN + u] = ldg16(vp + src_off(c_next, u, row0));
+            *(u32x4_t FCK_LDS*)(vstage + vw_off[u]) = staged(f.a[S::VN + u]);
+            f.a[S::VN + u] = fetch(vp + src_off(c_next, u, row0));
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -451,7 +474,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
                 }
                 const int i = r / g, h = (hkv0 + hl) * g + r % g;
                 const int64_t wofs = ((int64_t)(wb * a.hq + h) * a.num_splits + split) * Sq + wrow0 + i;
-                o_acc[wofs * D + c] = (L == 0.f) ? 0.f : acc / L;
+                o_acc[wofs * D + c] = (L == 0.f) ? 0.f : acc / L * a.v_descale;
                 if (c == 0) lse_acc[wofs] = (L == 0.f) ? -INFINITY : (mmax + fast_log2(L)) * kLn2;
             }
         }
@@ -526,9 +549,17 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
     constexpr size_t lds = decode_lds_bytes<D, NW, HG>();
     if constexpr (HG == 1) {
         if (a.mod.active()) {
+            if (a.kv8) {
+                if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true, true>>(grid, block, lds, st, a);
+                return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true, true>>(grid, block, lds, st, a);
+            }
             if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true>>(grid, block, lds, st, a);
             return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true>>(grid, block, lds, st, a);
         }
+    }
+    if (a.kv8) {
+        if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, false, true>>(grid, block, lds, st, a);
+        return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, false, true>>(grid, block, lds, st, a);
     }
     if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true>>(grid, block, lds, st, a);
     return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false>>(grid, block, lds, st, a);

@@ -164,9 +164,10 @@ def workload_varlen_prefill(seed=BASE_SEED + 5, batch=16, hq=32, hk=8, head_dim=
 # algorithmic work of a call (what the roofline figures are computed from)
 # ---------------------------------------------------------------------------------------------------------------
 
-def decode_bytes(lens, q_lens, hq, hk, d, dv, page_size, elem=2):
-    """K and V once, Q in, O out, block-table entries and sequence lengths; fp32 workspace traffic excluded."""
-    kv = sum(lens) * hk * (d + dv) * elem
+def decode_bytes(lens, q_lens, hq, hk, d, dv, page_size, elem=2, kv_elem=None):
+    """K and V once, Q in, O out, block-table entries and sequence lengths; fp32 workspace traffic excluded.
+    kv_elem: bytes per K/V element when the cache type differs from the Q/O type (1 for an fp8 cache)."""
+    kv = sum(lens) * hk * (d + dv) * (elem if kv_elem is None else kv_elem)
     qo = sum(q_lens) * hq * (d + dv) * elem
     idx = 4 * (sum(-(-l // page_size) for l in lens) + len(lens))
     return kv + qo + idx

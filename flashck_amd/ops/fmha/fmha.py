@@ -122,7 +122,7 @@ def _window(window):
     return int(wl), int(wr)
 
 
-def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols):
+def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols, kv_fp8=False, k_descale=1.0, v_descale=1.0):
     """fck_fmha_attrs for a call, or None when no score modifier is asked for.
 
     bias (elementwise, BiasEnum ELEMENTWISE_BIAS): q's dtype, last dim contiguous; batch mode [1|B, 1|Hq, sq, >= sk],
@@ -132,13 +132,17 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols)
     cap = float(logits_soft_cap)
     if not (cap >= 0.0) or math.isinf(cap):
         raise ValueError("logits_soft_cap must be finite and >= 0")
-    if bias is None and alibi_slopes is None and cap == 0.0:
+    if bias is None and alibi_slopes is None and cap == 0.0 and not kv_fp8:
         return None, None
     if bias is not None and alibi_slopes is not None:
         raise ValueError("bias and alibi_slopes are exclusive (one BiasEnum per call)")
     a = _lib.Attrs()
     a.size = ctypes.sizeof(_lib.Attrs)
     a.logits_soft_cap = cap
+    if kv_fp8:
+        if not (float(k_descale) > 0.0 and float(v_descale) > 0.0 and math.isfinite(k_descale) and math.isfinite(v_descale)):
+            raise ValueError("k_descale and v_descale must be positive and finite")
+        a.kv_dtype, a.k_descale, a.v_descale = 1, float(k_descale), float(v_descale)  # flashck::DataType FLOAT8
     Hq = q.shape[-2]
     if bias is not None:
         if not isinstance(bias, torch.Tensor):
@@ -250,16 +254,18 @@ def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scal
 def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=None, cache_batch_idx=None,
                      cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q: int = 0, scale: float = 0.0,
                      mask_type: int = MASK_NONE, window=(-1, -1), o_acc=None, lse_acc=None, bias=None, alibi_slopes=None,
-                     logits_soft_cap: float = 0.0):
+                     logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0):
     """Split-KV forward: returns the per-split partials (o_acc, lse_acc), to be merged by fmha_fwd_splitkv_combine.
-    bias / alibi_slopes / logits_soft_cap: see _attrs.
+    bias / alibi_slopes / logits_soft_cap: see _attrs.  k and v may be torch.float8_e4m3fn (a quantised cache with the
+    static per-tensor scales k_descale, v_descale: value = descale * stored); q and the output keep q's dtype.
 
     k/v are a paged cache when block_table is given, packed when cu_seqlens_k is given, else [B*, sk, Hk, D].
     """
     group = cu_seqlens_q is not None
     _check_tensor("q", q, ndim=3 if group else 4)
-    _check_tensor("k", k, dtype=q.dtype)
-    _check_tensor("v", v, dtype=q.dtype)
+    kv_fp8 = isinstance(k, torch.Tensor) and k.dtype == torch.float8_e4m3fn
+    _check_tensor("k", k, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype)
+    _check_tensor("v", v, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype)
     for name, t in (("seqlen_k", seqlen_k), ("block_table", block_table), ("cache_batch_idx", cache_batch_idx),
                     ("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
         _check_tensor(name, t, dtype=torch.int32, optional=True)
@@ -297,7 +303,8 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
         _check_shape("o_acc", o_acc, (bs, Hq, int(num_splits), sq, Dv), q)
         _check_shape("lse_acc", lse_acc, (bs, Hq, int(num_splits), sq), q)
     wl, wr = _window(window)
-    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, sq, 1 if (group or block_table is not None) else sk)
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, sq, 1 if (group or block_table is not None) else sk,
+                      kv_fp8, k_descale, v_descale)
     if at is None:
         _call("fck_fmha_fwd_splitkv", _ptr(q), _ptr(k), _ptr(v), None, _ptr(lse_acc), _ptr(o_acc), _ptr(cu_seqlens_q),
               _ptr(cu_seqlens_k), _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv,

@@ -37,6 +37,7 @@ extern "C" {
 #define FCK_EXPORT __attribute__((visibility("default")))
 
 /* flashck::DataType, core/utils/dtype.h:16-28 */
+#define FCK_DTYPE_FP8 1 /* e4m3 (OCP, as ck_tile::fp8_t on gfx950); accepted as fck_fmha_attrs.kv_dtype only */
 #define FCK_DTYPE_FP16 3
 #define FCK_DTYPE_BF16 4
 
@@ -63,6 +64,9 @@ extern "C" {
  * (core/profiling/attention/fmha_fwd_split_kv/fmha_fwd_split_kv_problem.h:81).  Passed to the *_attrs entry points;
  * a NULL pointer (or the entry point without the suffix) means none of them.
  *
+ * and static quantisation (is_static_quant, same file :79; fp8 type roles
+ * core/module/kernels/attention_kernels/fmha_common_jinja.h:157-171).
+ *
  * Scores: x = scale * q.k;  x = cap * tanh(x / cap) when logits_soft_cap > 0;  x += bias;  then the mask.
  *   ELEMENTWISE_BIAS  T elements; (b, h, i, j) at bias[b * bias_batch_stride + h * bias_head_stride + i * bias_row_stride + j].
  *                     The reference's rank 0 (1*1*s*s) is head and batch stride 0, rank 1 (1*h*s*s) batch stride 0,
@@ -81,7 +85,11 @@ typedef struct fck_fmha_attrs {
     int64_t bias_head_stride;
     int64_t bias_row_stride;
     float logits_soft_cap;     /* > 0: on; 0: off */
-    uint32_t reserved;         /* 0 */
+    /* K/V cache element type when it differs from `dtype`: 0 = same as Q, FCK_DTYPE_FP8 = one e4m3 byte per element
+     * with static per-tensor scales (split-KV entry point only): k = k_descale * fp8 value, v = v_descale * fp8 value;
+     * Q, the probabilities and the output keep `dtype`.  A descale of 0 means 1. */
+    int32_t kv_dtype;
+    float k_descale, v_descale;
 } fck_fmha_attrs;
 
 #define FCK_OK 0

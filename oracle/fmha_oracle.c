@@ -97,6 +97,21 @@ static inline uint16_t f32_to_fp16(float f)
     return (uint16_t)(sign | h);
 }
 
+/* OCP e4m3 ("e4m3fn"): 1 sign, 4 exponent (bias 7), 3 mantissa bits; no infinities, S.1111.111 is NaN, exponent 0 is
+   subnormal (mantissa / 8 * 2^-6). */
+float fck_orc_fp8_to_f32(uint8_t x)
+{
+    const int e = (x >> 3) & 15, m = x & 7;
+    float v;
+    if (e == 15 && m == 7)
+        v = NAN;
+    else if (e == 0)
+        v = ldexpf((float)m, -9);
+    else
+        v = ldexpf(1.f + (float)m / 8.f, e - 7);
+    return (x & 0x80) ? -v : v;
+}
+
 static inline float ld(const void* base, int64_t idx, int dtype)
 {
     uint16_t x = ((const uint16_t*)base)[idx];
@@ -224,6 +239,8 @@ static void attend_row(const fck_orc_problem* p, const void* q, const void* k, c
     mask_coords(p->mask_type, p->window_left, p->window_right, sq_b, sk_b, &y, &x);
     for (int t = 0; t < d; ++t) sc->qf[t] = ld(q, (qrow * p->hq + h) * d + t, dt);
 
+    const int kv8 = p->kv_dtype == FCK_ORC_FP8;
+    const float kd = (kv8 && p->k_descale != 0.f) ? p->k_descale : 1.f, vd = (kv8 && p->v_descale != 0.f) ? p->v_descale : 1.f;
     /* bias row of (b, h, i) / ALiBi slope of (b, h) */
     int64_t bias_row = 0;
     float slope = 0.f;
@@ -247,8 +264,11 @@ static void attend_row(const fck_orc_problem* p, const void* q, const void* k, c
     for (int j = k0; j < k1; ++j) {
         float acc = 0.f;
         const int64_t base = (rows[j] * hk + hkv) * d;
-        for (int t = 0; t < d; ++t) acc += sc->qf[t] * ld(k, base + t, dt);
-        float sv = acc * p->scale;
+        if (kv8)
+            for (int t = 0; t < d; ++t) acc += sc->qf[t] * fck_orc_fp8_to_f32(((const uint8_t*)k)[base + t]);
+        else
+            for (int t = 0; t < d; ++t) acc += sc->qf[t] * ld(k, base + t, dt);
+        float sv = acc * (p->scale * kd);
         if (p->logits_soft_cap > 0.f) sv = p->logits_soft_cap * tanhf(sv / p->logits_soft_cap);
         if (p->bias_type == 1) {
             sv += ld(p->bias, bias_row + j, dt);
@@ -273,8 +293,12 @@ static void attend_row(const fck_orc_problem* p, const void* q, const void* k, c
         float pj = rnd(expf(sc->s[j - k0] - vmax) * inv, dt);
         if (pj == 0.f) continue; /* masked keys may sit in pages holding non-finite fill */
         const int64_t base = (rows[j] * hk + hkv) * dv;
-        for (int t = 0; t < dv; ++t) sc->of[t] += pj * ld(v, base + t, dt);
+        if (kv8)
+            for (int t = 0; t < dv; ++t) sc->of[t] += pj * fck_orc_fp8_to_f32(((const uint8_t*)v)[base + t]);
+        else
+            for (int t = 0; t < dv; ++t) sc->of[t] += pj * ld(v, base + t, dt);
     }
+    for (int t = 0; t < dv; ++t) sc->of[t] *= vd;
     /* softmax reference: lse = max + ln(sum); a row with no visible key gives ln(0) = -inf */
     *lse_out = (sum == 0.f) ? -INFINITY : vmax + logf(sum);
 }

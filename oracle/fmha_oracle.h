@@ -19,7 +19,7 @@ extern "C" {
 #endif
 
 /* flashck::DataType ids, core/utils/dtype.h:16-28 */
-enum { FCK_ORC_FP16 = 3, FCK_ORC_BF16 = 4 };
+enum { FCK_ORC_FP8 = 1, FCK_ORC_FP16 = 3, FCK_ORC_BF16 = 4 };
 
 /* GenericAttentionMaskEnum, core/profiling/attention/fmha_library.h:81-87 */
 enum { FCK_ORC_NO_MASK = 0, FCK_ORC_MASK_TOP_LEFT = 1, FCK_ORC_MASK_BOTTOM_RIGHT = 2, FCK_ORC_MASK_GENERIC = 3 };
@@ -70,6 +70,12 @@ typedef struct {
     const void* bias;
     int64_t bias_batch_stride, bias_head_stride, bias_row_stride;
     float logits_soft_cap;
+    /* K/V element type when it is not `dtype`: FCK_ORC_FP8 = one e4m3 byte per element (the OCP format ck_tile::fp8_t
+       is on gfx950, ck_tile/core/numeric/float8.hpp) with static per-tensor scales: k = k_descale * value,
+       v = v_descale * value (0 means 1).  Type roles: core/module/kernels/attention_kernels/fmha_common_jinja.h:157-171;
+       is_static_quant: core/profiling/attention/fmha_fwd_split_kv/fmha_fwd_split_kv_problem.h:79. */
+    int32_t kv_dtype;
+    float k_descale, v_descale;
 } fck_orc_problem;
 
 /* 1 when key j is visible to query i. */
@@ -103,6 +109,9 @@ int fck_orc_appendkv(void* q, void* k_cache, void* v_cache, const void* knew, co
 /* Gather one sequence's first n rows of a paged cache into dst [n, Hk, D]. */
 int fck_orc_gather_paged(const void* cache, const int32_t* pages, int page_size, int n, int hk, int d,
                          int elem_bytes, void* dst);
+
+/* value of one e4m3 byte (NaN for 0x7f / 0xff) */
+float fck_orc_fp8_to_f32(uint8_t x);
 
 int fck_orc_num_threads(void);
 

@@ -12,7 +12,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libfmha_oracle.so")
 
-FP16, BF16 = 3, 4
+FP8, FP16, BF16 = 1, 3, 4
 NO_MASK, MASK_TOP_LEFT, MASK_BOTTOM_RIGHT, MASK_GENERIC = 0, 1, 2, 3
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALF_ROTATED = 0, 1, 2
 KV_BATCH, KV_GROUP, KV_BLOCK_TABLE, KV_PAGE_LIST = 0, 1, 2, 3
@@ -45,6 +45,7 @@ class _Problem(ctypes.Structure):
         ("bias", ctypes.c_void_p),
         ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64),
         ("logits_soft_cap", ctypes.c_float),
+        ("kv_dtype", ctypes.c_int32), ("k_descale", ctypes.c_float), ("v_descale", ctypes.c_float),
     ]
 
 
@@ -72,6 +73,12 @@ def lib():
                                           ctypes.c_int, ctypes.c_void_p, ctypes.c_int64] + [ctypes.c_int] * 6)
         _lib.fck_orc_gather_paged.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 5 + [ctypes.c_void_p]
     return _lib
+
+
+def fp8_to_f32(byte: int) -> float:
+    lib().fck_orc_fp8_to_f32.restype = ctypes.c_float
+    lib().fck_orc_fp8_to_f32.argtypes = [ctypes.c_uint8]
+    return lib().fck_orc_fp8_to_f32(byte)
 
 
 def num_threads():
@@ -102,7 +109,8 @@ def _i32(t):
 
 def _problem(q, k, v, *, seqstart_q=None, seqstart_k=None, seqlen_k=None, block_table=None, page_size=0,
              kv_indptr=None, kv_page_indices=None, kv_last_page_lens=None, cache_batch_idx=None, scale=None,
-             mask_type=NO_MASK, window=(-1, -1), batch=None, bias=None, alibi_slopes=None, logits_soft_cap=0.0):
+             mask_type=NO_MASK, window=(-1, -1), batch=None, bias=None, alibi_slopes=None, logits_soft_cap=0.0,
+             k_descale=1.0, v_descale=1.0):
     """bias: data dtype, [1|B, 1|Hq, sq, sk] (batch mode) or [1|Hq, total_q, max_sk] (group mode), last dim contiguous;
     alibi_slopes: fp32 [Hq] or [B, Hq]; logits_soft_cap > 0: s = cap * tanh(scale * qk / cap)."""
     p = _Problem()
@@ -142,6 +150,9 @@ def _problem(q, k, v, *, seqstart_q=None, seqstart_k=None, seqlen_k=None, block_
     p.mask_type = int(mask_type)
     p.window_left, p.window_right = int(window[0]), int(window[1])
     p.logits_soft_cap = float(logits_soft_cap)
+    if k.dtype == torch.float8_e4m3fn:   # fp8 K/V with static scales
+        assert v.dtype == torch.float8_e4m3fn
+        p.kv_dtype, p.k_descale, p.v_descale = FP8, float(k_descale), float(v_descale)
     assert bias is None or alibi_slopes is None, "one bias kind at a time"
     if bias is not None:
         assert bias.dtype == q.dtype and bias.device.type == "cpu" and bias.stride(-1) == 1

@@ -183,3 +183,63 @@ def test_modifier_arguments_are_validated(fmha):
                           4, 0.125, -1, -1, 0, 3, None)
     assert rc == -2 and b"fck_fmha_attrs" in lib.fck_last_error()
     del ctypes
+
+
+def quantise_cache(kv, k_descale, v_descale):
+    """fp8 (e4m3) copies of a paged cache with static per-tensor scales; unused slots stay NaN"""
+    k8 = (kv["k_cache"].float() / k_descale).to(torch.float8_e4m3fn)
+    v8 = (kv["v_cache"].float() / v_descale).to(torch.float8_e4m3fn)
+    return k8, v8
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hk,d,page,ns,batch", [(8, 2, 128, 128, 3, 3), (32, 8, 128, 128, 4, 20), (16, 8, 64, 64, 2, 3),
+                                                   (4, 4, 256, 64, 2, 2), (8, 2, 128, 48, 2, 3)])
+def test_paged_decode_fp8_cache(fmha, orc, dtype, hq, hk, d, page, ns, batch):
+    """K/V stored as e4m3 bytes with static scales; q, the probabilities and the output keep the 16-bit type.  The
+    20-sequence case fills the grid, so it takes the two-heads-per-workgroup variant; page 48 the per-row lookup."""
+    w = gen.workload_paged_decode(seed=91 + hq + d, batch=batch, hq=hq, hk=hk, head_dim=d, min_len=1, max_len=600, page_size=page,
+                                  dtype=dtype)
+    kd, vd = 0.03, 0.025
+    k8, v8 = quantise_cache(w, kd, vd)
+    q, bt, sl = dev(w["q"]), dev(w["block_table"]), dev(w["seqlen_k"])
+    o_acc, lse_acc = fmha.fmha_fwd_splitkv(q, dev(k8), dev(v8), ns, seqlen_k=sl, block_table=bt, scale=w["scale"], k_descale=kd,
+                                           v_descale=vd)
+    assert b"kv_fp8" in _lib.load().fck_fmha_last_kernel()
+    o = fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype)
+    torch.cuda.synchronize()
+    kw = dict(seqlen_k=w["seqlen_k"], block_table=w["block_table"], scale=w["scale"], k_descale=kd, v_descale=vd)
+    ro_acc, rlse_acc = orc.fmha_splitkv(w["q"], k8, v8, ns, **kw)
+    ro = orc.fmha_fwd(w["q"], k8, v8, **kw)
+    assert_lse_close(lse_acc, rlse_acc, what="lse_acc")
+    assert_close(o_acc, ro_acc, ATOL[dtype], "o_acc")
+    assert_close(o, ro, ATOL[dtype], "o")
+
+
+def test_multi_query_decode_fp8_cache_with_alibi(fmha, orc):
+    g = torch.Generator().manual_seed(95)
+    dtype, sq, hq, hk, d = torch.bfloat16, 6, 8, 2, 128
+    lens = [6, 70, 200]
+    kv = gen.paged_kv(lens, hk, d, dtype, g, 64)
+    k8, v8 = quantise_cache(kv, 0.04, 0.04)
+    qh = gen.randn((3, sq, hq, d), dtype, g)
+    okw, dkw = mods("alibi_h", dtype, g, 3, hq, sq, max(lens))
+    scale = 1 / math.sqrt(d)
+    o_acc, lse_acc = fmha.fmha_fwd_splitkv(dev(qh), dev(k8), dev(v8), 2, seqlen_k=dev(kv["seqlen_k"]), block_table=dev(kv["block_table"]),
+                                           scale=scale, mask_type=2, window=(-1, 0), k_descale=0.04, v_descale=0.04, **dkw)
+    o = fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype)
+    torch.cuda.synchronize()
+    ro = orc.fmha_fwd(qh, k8, v8, seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], scale=scale, mask_type=2, window=(-1, 0),
+                      k_descale=0.04, v_descale=0.04, **okw)
+    assert_close(o, ro, ATOL[dtype], "o")
+
+
+def test_fp8_cache_is_refused_where_no_kernel_reads_it(fmha):
+    import ctypes
+    lib = _lib.load()
+    at = _lib.Attrs()
+    at.size, at.kv_dtype = ctypes.sizeof(_lib.Attrs), 1
+    x = torch.zeros(1, 4, 4, 64, dtype=torch.float16, device="cuda")
+    rc = lib.fck_fmha_fwd_attrs(x.data_ptr(), x.data_ptr(), x.data_ptr(), None, x.data_ptr(), None, None, None, 1, 4, 4, 4, 4, 64, 64,
+                                4, 0.125, -1, -1, 0, 3, ctypes.byref(at), None)
+    assert rc == -2 and b"split-KV entry point only" in lib.fck_last_error()

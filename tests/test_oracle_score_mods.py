@@ -136,3 +136,32 @@ def test_split_kv_partials_carry_the_modifiers(orc):
         o_acc, lse_acc = orc.fmha_splitkv(q, k, v, 4, mask_type=2, window=(-1, 0), **kw)
         merged = orc.splitkv_combine(lse_acc, o_acc, dtype).float()
         assert (merged - whole).abs().max() <= 1.6e-2
+
+
+def test_fp8_byte_values_match_the_library_type(orc):
+    """Every e4m3 byte decodes to what torch.float8_e4m3fn (the OCP format) says it is."""
+    ref = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float()
+    for byte in range(256):
+        got = orc.fp8_to_f32(byte)
+        assert (math.isnan(got) and math.isnan(ref[byte].item())) or got == ref[byte].item(), byte
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)])
+def test_fp8_kv_matches_sdpa_on_the_dequantised_cache(orc, dtype, tol):
+    g = torch.Generator().manual_seed(13)
+    B, sq, sk, hq, hk, d = 2, 3, 77, 4, 2, 64
+    kd, vd = 0.05, 0.02
+    q = gen.randn((B, sq, hq, d), dtype, g)
+    k8 = (gen.randn((B, sk, hk, d), torch.float32, g) / kd).to(torch.float8_e4m3fn)
+    v8 = (gen.randn((B, sk, hk, d), torch.float32, g) / vd).to(torch.float8_e4m3fn)
+    o, lse = orc.fmha_fwd(q, k8, v8, return_lse=True, mask_type=2, window=(-1, 0), k_descale=kd, v_descale=vd)
+    kf, vf = k8.float() * kd, v8.float() * vd
+    vis = flash_mask(2, (-1, 0), sq, sk)
+    ref = sdpa(q.float(), kf, vf, mask=vis)
+    assert (o.float() - ref).abs().max() <= tol
+    s = torch.einsum("bqhd,bkhd->bhqk", q.float(), kf.repeat_interleave(hq // hk, 2)) / math.sqrt(d)
+    s = s.masked_fill(~vis, float("-inf"))
+    assert (lse - torch.logsumexp(s, -1)).abs().max() <= 1e-4
+    # the split partials merge to the same result
+    o_acc, lse_acc = orc.fmha_splitkv(q, k8, v8, 3, mask_type=2, window=(-1, 0), k_descale=kd, v_descale=vd)
+    assert (orc.splitkv_combine(lse_acc, o_acc, dtype).float() - o.float()).abs().max() <= tol
