@@ -60,6 +60,7 @@ def parse():
     ap.add_argument("--kv-len", type=int, default=32768, help="KV length of the split-KV workload (study runs only)")
     ap.add_argument("--no-shuffle", action="store_true", help="identity page order (study runs only)")
     ap.add_argument("--num-splits", type=int, default=8, help="split count of the split-KV workload (study runs only)")
+    ap.add_argument("--paged-splits", type=int, default=0, help="split count of the paged-decode workload (0: the library's heuristic)")
     ap.add_argument("--kv-fp8", action="store_true", help="split-KV workload with the cache stored as fp8 (e4m3, static scales)")
     ap.add_argument("--decode-path", default="two-launch", choices=["two-launch", "fused"],
                     help="two-launch: split-KV + combine kernels with a caller-owned workspace; fused: one launch "
@@ -119,7 +120,7 @@ def bench_decode(args, torch, fmha, gen, which):
             ns = 0
             name = "paged-KV decode: B=32 q=1 Hq32/Hk8 D128 L~U[512,4096] P=128, one fused launch, library-chosen ranges (bf16)"
         else:
-            ns = fmha.num_splits_heuristic(32, 32, 8, 1, max(w["lens"]), 128)
+            ns = args.paged_splits or fmha.num_splits_heuristic(32, 32, 8, 1, max(w["lens"]), 128)
             name = f"paged-KV decode: B=32 q=1 Hq32/Hk8 D128 L~U[512,4096] P=128 ns={ns} + combine (bf16)"
     B, _, Hq, D = w["q"].shape
     Hk = w["k_cache"].shape[2]

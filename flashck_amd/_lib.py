@@ -17,7 +17,7 @@ class Attrs(ctypes.Structure):
     _fields_ = [("size", ctypes.c_uint32), ("bias_type", ctypes.c_int32), ("bias", ctypes.c_void_p),
                 ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64),
                 ("logits_soft_cap", ctypes.c_float), ("kv_dtype", ctypes.c_int32), ("k_descale", ctypes.c_float),
-                ("v_descale", ctypes.c_float)]
+                ("v_descale", ctypes.c_float), ("decode_variant", ctypes.c_int32)]
 
 
 _ap = ctypes.POINTER(Attrs)

@@ -199,6 +199,14 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
     a.v_descale = 1.f;
+    if (attrs && attrs->decode_variant != 0) {
+        if (attrs->decode_variant != 1 && attrs->decode_variant != 2)
+            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant %d out of range [0,2]", attrs->decode_variant);
+        if (attrs->decode_variant == 2 && (hk % 2 || d > 128 || q_max_seq_len * (hq / hk) > 16 || a.mod.active()))
+            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant 2 (head pairs) needs an even kv_num_heads, head dim <= 128, at most 16 packed "
+                                                  "query rows and no bias / soft cap");
+        a.variant = attrs->decode_variant;
+    }
     if (attrs && attrs->kv_dtype != 0) {
         // fp8 K/V with static per-tensor scales: the K scale multiplies every score, the V scale the output
         if (attrs->kv_dtype != FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: only 0 (same as q) and FLOAT8 (1)", attrs->kv_dtype);

@@ -45,6 +45,7 @@ struct SplitKvArgs {
     uint32_t mask_type;
     int64_t window_left, window_right;
     ScoreMod mod;      // bias / ALiBi / soft cap; all zero: none
+    int32_t variant;   // 0: chosen by the launcher; 1: one KV head per workgroup; 2: head pairs
     int32_t kv8;       // K and V are fp8 (e4m3); the K scale is folded into scale_log2 / mod.scale by the caller
     float v_descale;   // factor on the output (1 unless V is quantised)
 };

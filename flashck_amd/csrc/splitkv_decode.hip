@@ -569,6 +569,7 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
 // covers the CUs.
 static bool use_head_pairs(const SplitKvArgs& a, int m_tiles, int num_cu)
 {
+    if (a.variant != 0) return a.variant == 2;  // validated by the caller
     if (a.hk % 2 || a.mod.active()) return false;
     return (int64_t)(a.hk / 2) * a.num_splits * m_tiles * a.batch >= num_cu;
 }

@@ -122,7 +122,8 @@ def _window(window):
     return int(wl), int(wr)
 
 
-def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols, kv_fp8=False, k_descale=1.0, v_descale=1.0):
+def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols, kv_fp8=False, k_descale=1.0, v_descale=1.0,
+           decode_variant=0):
     """fck_fmha_attrs for a call, or None when no score modifier is asked for.
 
     bias (elementwise, BiasEnum ELEMENTWISE_BIAS): q's dtype, last dim contiguous; batch mode [1|B, 1|Hq, sq, >= sk],
@@ -132,13 +133,16 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
     cap = float(logits_soft_cap)
     if not (cap >= 0.0) or math.isinf(cap):
         raise ValueError("logits_soft_cap must be finite and >= 0")
-    if bias is None and alibi_slopes is None and cap == 0.0 and not kv_fp8:
+    if int(decode_variant) not in (0, 1, 2):
+        raise ValueError("decode_variant must be 0 (library's choice), 1 (one KV head per workgroup) or 2 (head pairs)")
+    if bias is None and alibi_slopes is None and cap == 0.0 and not kv_fp8 and not decode_variant:
         return None, None
     if bias is not None and alibi_slopes is not None:
         raise ValueError("bias and alibi_slopes are exclusive (one BiasEnum per call)")
     a = _lib.Attrs()
     a.size = ctypes.sizeof(_lib.Attrs)
     a.logits_soft_cap = cap
+    a.decode_variant = int(decode_variant)
     if kv_fp8:
         if not (float(k_descale) > 0.0 and float(v_descale) > 0.0 and math.isfinite(k_descale) and math.isfinite(v_descale)):
             raise ValueError("k_descale and v_descale must be positive and finite")
@@ -254,8 +258,10 @@ def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scal
 def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=None, cache_batch_idx=None,
                      cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q: int = 0, scale: float = 0.0,
                      mask_type: int = MASK_NONE, window=(-1, -1), o_acc=None, lse_acc=None, bias=None, alibi_slopes=None,
-                     logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0):
+                     logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0, decode_variant: int = 0):
     """Split-KV forward: returns the per-split partials (o_acc, lse_acc), to be merged by fmha_fwd_splitkv_combine.
+    decode_variant: 0 = the library picks the kernel variant, 1 / 2 force it (what the tuner records, see
+    tune_decode_num_splits).
     bias / alibi_slopes / logits_soft_cap: see _attrs.  k and v may be torch.float8_e4m3fn (a quantised cache with the
     static per-tensor scales k_descale, v_descale: value = descale * stored); q and the output keep q's dtype.
 
@@ -304,7 +310,7 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
         _check_shape("lse_acc", lse_acc, (bs, Hq, int(num_splits), sq), q)
     wl, wr = _window(window)
     at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, sq, 1 if (group or block_table is not None) else sk,
-                      kv_fp8, k_descale, v_descale)
+                      kv_fp8, k_descale, v_descale, decode_variant)
     if at is None:
         _call("fck_fmha_fwd_splitkv", _ptr(q), _ptr(k), _ptr(v), None, _ptr(lse_acc), _ptr(o_acc), _ptr(cu_seqlens_q),
               _ptr(cu_seqlens_k), _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv,
@@ -534,9 +540,10 @@ def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q
     return o
 
 
-def _auto_num_splits(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size, dtype) -> int:
-    """A tuned split count recorded for this class of problems if there is one, else the heuristic."""
-    return tuning.choose_num_splits(
+def _auto_num_splits(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size, dtype):
+    """(split count, kernel variant): the tuned pair recorded for this class of problems if there is one, else the
+    heuristic split count and variant 0 (the library's choice)."""
+    return tuning.choose_splitkv(
         lambda: num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim),
         batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size,
         "fp16" if dtype == torch.float16 else "bf16")
@@ -544,21 +551,27 @@ def _auto_num_splits(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, h
 
 def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits: int = 0, max_seqlen_k: int = 0,
                       cu_seqlens_q=None, max_seqlen_q: int = 0, scale: float = 0.0, mask_type: int = MASK_NONE,
-                      window=(-1, -1), workspace=None, out=None, fused: bool = False) -> torch.Tensor:
-    """Paged decode = split-KV forward + LSE combine; num_splits = 0 asks the heuristic (needs max_seqlen_k).
+                      window=(-1, -1), workspace=None, out=None, fused: bool = False, bias=None, alibi_slopes=None,
+                      logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0,
+                      decode_variant: int = 0) -> torch.Tensor:
+    """Paged decode = split-KV forward + LSE combine; num_splits = 0 asks the tuning cache, then the heuristic (needs
+    max_seqlen_k); a cached record also brings the kernel variant it was measured with.  bias / alibi_slopes /
+    logits_soft_cap / fp8 caches with k_descale, v_descale: as fmha_fwd_splitkv (not with fused = True).
 
     fused = True runs both in one launch that allocates nothing (fmha_fwd_splitkv_fused; the partial results then live
     in the library's fixed device array, `workspace` is not used, and problems beyond its limits raise)."""
     group = cu_seqlens_q is not None
     _check_tensor("q", q, ndim=3 if group else 4)
-    _check_tensor("k_cache", k_cache, dtype=q.dtype, ndim=4)
-    _check_tensor("v_cache", v_cache, dtype=q.dtype, ndim=4)
+    kv_fp8 = isinstance(k_cache, torch.Tensor) and k_cache.dtype == torch.float8_e4m3fn
+    _check_tensor("k_cache", k_cache, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype, ndim=4)
+    _check_tensor("v_cache", v_cache, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype, ndim=4)
     _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1)
     _check_tensor("block_table", block_table, dtype=torch.int32, ndim=2)
     Hq, D = q.shape[-2], q.shape[-1]
     Hk = k_cache.shape[2]
     B = seqlen_k.numel()
     sq = max_seqlen_q if group else q.shape[1]
+    plain = bias is None and alibi_slopes is None and not logits_soft_cap and not kv_fp8
     if workspace is not None and num_splits <= 0:
         # the partials are laid out for one split count: with a caller-owned workspace that count is the workspace's
         num_splits = int(workspace[0].shape[2]) if workspace[0].dim() == 5 else 0
@@ -567,23 +580,30 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
     if num_splits <= 0:
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * k_cache.shape[1]
-        num_splits = _auto_num_splits(B, Hq, Hk, sq, max_seqlen_k, D, k_cache.shape[1], q.dtype)
+        num_splits, cached_variant = _auto_num_splits(B, Hq, Hk, sq, max_seqlen_k, D, k_cache.shape[1], q.dtype)
+        if not decode_variant and plain:
+            decode_variant = cached_variant
     if fused:
+        if not plain or decode_variant:
+            raise NotImplementedError("the fused launch takes no bias / soft cap / fp8 cache / kernel variant")
         return fmha_fwd_splitkv_fused(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_k, block_table=block_table,
                                       cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, scale=scale,
                                       mask_type=mask_type, window=window, out=out)
     o_acc, lse_acc = workspace if workspace is not None else (None, None)
     o_acc, lse_acc = fmha_fwd_splitkv(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_k, block_table=block_table,
                                       cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, scale=scale,
-                                      mask_type=mask_type, window=window, o_acc=o_acc, lse_acc=lse_acc)
+                                      mask_type=mask_type, window=window, o_acc=o_acc, lse_acc=lse_acc, bias=bias,
+                                      alibi_slopes=alibi_slopes, logits_soft_cap=logits_soft_cap, k_descale=k_descale,
+                                      v_descale=v_descale, decode_variant=decode_variant)
     return fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, out=out)
 
 
 def tune_decode_num_splits(q, k_cache, v_cache, seqlen_k, block_table, *, max_seqlen_k: int,
-                           candidates=(1, 2, 4, 8, 16, 32, 64), **kwargs) -> dict:
-    """Time `fmha_decode_paged` with each candidate split count on these tensors and record the fastest for the
-    problem class (see utils/tuning.py); later calls with num_splits = 0 on problems of that class use it.
-    Returns the record ({"num_splits", "latency_us", "tried_us", ...})."""
+                           candidates=(1, 2, 4, 8, 16, 32, 64), variants=(0,), **kwargs) -> dict:
+    """Time `fmha_decode_paged` with each candidate (split count, kernel variant) on these tensors and record the
+    fastest for the problem class (see utils/tuning.py); later calls with num_splits = 0 on problems of that class use
+    both.  variants: 0 = the library's own choice, 1 = one KV head per workgroup, 2 = head pairs (skipped where the
+    problem cannot take it).  Returns the record ({"num_splits", "variant", "kernel", "latency_us", "tried_us", ...})."""
     Hq, D = q.shape[-2], q.shape[-1]
     Hk, page = k_cache.shape[2], k_cache.shape[1]
     B = seqlen_k.numel()
@@ -591,14 +611,15 @@ def tune_decode_num_splits(q, k_cache, v_cache, seqlen_k, block_table, *, max_se
     problem = tuning.splitkv_problem(B, Hq, Hk, sq, max_seqlen_k, D, page, "fp16" if q.dtype == torch.float16 else "bf16")
     ws = {}
 
-    def run(ns):
+    def run(ns, variant=0):
         if ns not in ws:
             shape_batch, shape_sq = (1, q.shape[0]) if q.dim() == 3 else (q.shape[0], q.shape[1])
             ws[ns] = splitkv_workspace(shape_batch, Hq, shape_sq, v_cache.shape[3], ns, q.device)
         fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, num_splits=ns, max_seqlen_k=max_seqlen_k,
-                          workspace=ws[ns], **kwargs)
+                          workspace=ws[ns], decode_variant=variant, **kwargs)
+        return _lib.load().fck_fmha_last_kernel().decode()
 
-    return tuning.tune_num_splits(run, tuning.gpu_timer, candidates, problem)
+    return tuning.tune_num_splits(run, tuning.gpu_timer, candidates, problem, variants=variants)
 
 
 class DecodeWorkspace:
@@ -680,7 +701,9 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
     if num_splits <= 0:
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * page  # what the block table can address
-        num_splits = _auto_num_splits(B, Hq, Hk, n, max_seqlen_k, D, page, q.dtype)
+        num_splits, decode_variant = _auto_num_splits(B, Hq, Hk, n, max_seqlen_k, D, page, q.dtype)
+    else:
+        decode_variant = 0
     # a lone new token sees every key: no mask needed unless a sliding window is asked for
     if n == 1 and window_left < 0:
         mask_type, window = MASK_NONE, (-1, -1)
@@ -690,7 +713,7 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
     o_acc, lse_acc = ws.partials(shape_batch, Hq, num_splits, shape_sq, Dv, q.device)
     fmha_fwd_splitkv(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_new, block_table=block_table,
                      cu_seqlens_q=cu_seqlens_knew, max_seqlen_q=n if packed else 0, scale=scale, mask_type=mask_type,
-                     window=window, o_acc=o_acc, lse_acc=lse_acc)
+                     window=window, o_acc=o_acc, lse_acc=lse_acc, decode_variant=decode_variant)
     o = fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_knew, max_seqlen_q=n if packed else 0,
                                  out=out)
     return o, seqlen_new

@@ -17,7 +17,8 @@ from typing import Callable, Dict, Iterable, Optional
 
 from . import flags
 
-__all__ = ["TuningCache", "default_cache", "splitkv_problem", "choose_num_splits", "tune_num_splits", "environment"]
+__all__ = ["TuningCache", "default_cache", "splitkv_problem", "choose_num_splits", "choose_splitkv", "tune_num_splits",
+           "environment"]
 
 FILE_NAME = "flashck_amd_tuning.json"
 SCHEMA = 1
@@ -125,20 +126,32 @@ def default_cache() -> TuningCache:
 SPLITKV = "fmha_fwd_splitkv"
 
 
-def choose_num_splits(heuristic: Callable[[], int], batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim,
-                      page_size=0, dtype="bf16", cache: Optional[TuningCache] = None) -> int:
-    """Split count for a split-KV launch: a cached winner for the problem class when tuning is on, else `heuristic()`."""
+def choose_splitkv(heuristic: Callable[[], int], batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim,
+                   page_size=0, dtype="bf16", cache: Optional[TuningCache] = None):
+    """(split count, kernel variant) for a split-KV launch: the cached winner for the problem class when tuning is on,
+    else (`heuristic()`, 0 = the library picks the variant)."""
     if flags.flag("FC_TUNING_MODE") != 0:
         rec = (cache or default_cache()).query(
             SPLITKV, splitkv_problem(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size, dtype))
         if rec is not None and 1 <= int(rec.get("num_splits", 0)) <= 128:
-            return int(rec["num_splits"])
-    return int(heuristic())
+            variant = int(rec.get("variant", 0))
+            return int(rec["num_splits"]), (variant if variant in (0, 1, 2) else 0)
+    return int(heuristic()), 0
 
 
-def tune_num_splits(run: Callable[[int], None], timer: Callable[[Callable[[], None], int, int], float],
-                    candidates: Iterable[int], problem: str, nbytes: int = 0, cache: Optional[TuningCache] = None) -> dict:
-    """Measure `run(num_splits)` for every candidate and record the fastest for `problem`.
+def choose_num_splits(heuristic: Callable[[], int], batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim,
+                      page_size=0, dtype="bf16", cache: Optional[TuningCache] = None) -> int:
+    """Split count alone (see choose_splitkv)."""
+    return choose_splitkv(heuristic, batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size, dtype, cache)[0]
+
+
+def tune_num_splits(run: Callable[..., Optional[str]], timer: Callable[[Callable[[], None], int, int], float],
+                    candidates: Iterable[int], problem: str, nbytes: int = 0, cache: Optional[TuningCache] = None,
+                    variants: Iterable[int] = (0,)) -> dict:
+    """Measure `run(num_splits)` - with more than the default variant: `run(num_splits, variant)` - for every candidate
+    pair and record the fastest for `problem`, as ProfilingDB keeps (instance, split_k) per problem
+    (core/profiling/profiling_db.cc:64-71).  `run` may return the name of the kernel it launched; a pair the problem
+    cannot take (run raises ValueError / NotImplementedError) is skipped.
 
     `timer(fn, cold, repeats)` returns the mean seconds of one call of fn (on the GPU: events around `repeats` launches
     after `cold` untimed ones).  Returns the stored record.  An existing record is kept unless FC_FORCE_PROFILING is set.
@@ -151,18 +164,31 @@ def tune_num_splits(run: Callable[[int], None], timer: Callable[[Callable[[], No
     cold, repeats = flags.flag("FC_TUNING_NUM_COLD_ITERATION"), flags.flag("FC_TUNING_NUM_REPEATS")
     best = None
     tried = {}
+    variants = sorted(set(int(v) for v in variants)) or [0]
     for ns in sorted(set(int(c) for c in candidates)):
         if not 1 <= ns <= 128:
             continue
-        t = float(timer(lambda: run(ns), cold, repeats))
-        tried[str(ns)] = t * 1e6
-        if flags.flag("FC_TUNING_LOG"):
-            print(f"[flashck tuning] {problem}: num_splits={ns} {t * 1e6:.1f} us")
-        if best is None or t < best[1]:
-            best = (ns, t)
+        for variant in variants:
+            names = []
+
+            def call(ns=ns, variant=variant):
+                names.append(run(ns) if variants == [0] else run(ns, variant))
+
+            try:
+                t = float(timer(call, cold, repeats))
+            except (ValueError, NotImplementedError):
+                continue  # a variant this problem cannot take
+            kernel = names[-1] if names else None
+            tried[str(ns) if variants == [0] else f"{ns}/v{variant}"] = t * 1e6
+            if flags.flag("FC_TUNING_LOG"):
+                print(f"[flashck tuning] {problem}: num_splits={ns} variant={variant} {t * 1e6:.1f} us")
+            if best is None or t < best[1]:
+                best = (ns, t, variant, kernel)
     if best is None:
         raise ValueError("no valid num_splits candidate (1..128)")
-    rec = {"num_splits": best[0], "latency_us": best[1] * 1e6, "tried_us": tried}
+    rec = {"num_splits": best[0], "variant": best[2], "latency_us": best[1] * 1e6, "tried_us": tried}
+    if isinstance(best[3], str):
+        rec["kernel"] = best[3]
     if nbytes:
         rec["bandwidth_gbs"] = nbytes / best[1] / 1e9
     cache.insert(SPLITKV, problem, rec)

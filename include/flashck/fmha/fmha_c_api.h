@@ -90,6 +90,11 @@ typedef struct fck_fmha_attrs {
      * Q, the probabilities and the output keep `dtype`.  A descale of 0 means 1. */
     int32_t kv_dtype;
     float k_descale, v_descale;
+    /* Split-KV kernel variant, the counterpart of the tile instance FlashCK's tuner picks per problem
+     * (core/profiling/profiling_db.cc:64-71): 0 = the library chooses; 1 = one KV head per workgroup (32-key tiles);
+     * 2 = two adjacent KV heads per workgroup (16-key tiles, 512-byte row pieces; needs an even kv_num_heads, at most
+     * 16 packed query rows, head dim <= 128 and no bias / soft cap).  A variant the problem cannot take is an error. */
+    int32_t decode_variant;
 } fck_fmha_attrs;
 
 #define FCK_OK 0

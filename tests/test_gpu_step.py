@@ -103,6 +103,44 @@ def test_tuned_split_count_is_recorded_and_used(fmha, orc, tmp_path):
         tuning._default = old_default
 
 
+def test_decode_kernel_variant_is_tunable(fmha, orc, tmp_path):
+    """The two split-KV kernel variants (one KV head per workgroup, head pairs) forced through the attribute both match
+    the oracle; the tuner measures (split count, variant) pairs and a later num_splits = 0 call runs the recorded pair."""
+    import flashck_amd
+    from flashck_amd import _lib
+    from flashck_amd.utils import tuning
+    w = gen.workload_paged_decode(seed=76, batch=6, hq=16, hk=4, head_dim=128, min_len=300, max_len=1500, page_size=128)
+    q, kc, vc = dev(w["q"]), dev(w["k_cache"]), dev(w["v_cache"])
+    sl, bt = dev(w["seqlen_k"]), dev(w["block_table"])
+    ro = orc.fmha_fwd(w["q"], w["k_cache"], w["v_cache"], seqlen_k=w["seqlen_k"], block_table=w["block_table"], scale=w["scale"])
+    outs = {}
+    for variant in (1, 2):
+        outs[variant] = fmha.fmha_decode_paged(q, kc, vc, sl, bt, num_splits=2, scale=w["scale"], decode_variant=variant)
+        assert_close(outs[variant], ro, 2e-2, f"variant {variant}")
+    with pytest.raises(ValueError):   # head pairs need an even number of KV heads
+        odd = gen.workload_paged_decode(seed=77, batch=2, hq=6, hk=3, head_dim=128, min_len=50, max_len=100, page_size=128)
+        fmha.fmha_decode_paged(dev(odd["q"]), dev(odd["k_cache"]), dev(odd["v_cache"]), dev(odd["seqlen_k"]), dev(odd["block_table"]),
+                               num_splits=2, decode_variant=2)
+    saved = {n: flashck_amd.get_flag_value(n) for n in ("FC_TUNING_DB_DIR", "FC_TUNING_NUM_COLD_ITERATION",
+                                                          "FC_TUNING_NUM_REPEATS", "FC_TUNING_MODE")}
+    old_default = tuning._default
+    try:
+        flashck_amd.set_flag_value("FC_TUNING_DB_DIR", str(tmp_path))
+        flashck_amd.set_flag_value("FC_TUNING_NUM_COLD_ITERATION", "2")
+        flashck_amd.set_flag_value("FC_TUNING_NUM_REPEATS", "5")
+        flashck_amd.set_flag_value("FC_TUNING_MODE", "2")
+        tuning._default = None
+        rec = fmha.tune_decode_num_splits(q, kc, vc, sl, bt, max_seqlen_k=2048, candidates=(2, 4), variants=(1, 2), scale=w["scale"])
+        assert rec["variant"] in (1, 2) and set(rec["tried_us"]) == {"2/v1", "2/v2", "4/v1", "4/v2"}
+        assert rec["kernel"].startswith("splitkv_decode_kernel")
+        o = fmha.fmha_decode_paged(q, kc, vc, sl, bt, max_seqlen_k=2048, scale=w["scale"])   # num_splits = 0: the recorded pair
+        assert_close(o, ro, 2e-2, "decode with the tuned pair")
+    finally:
+        for n, v in saved.items():
+            flashck_amd.set_flag_value(n, v)
+        tuning._default = old_default
+
+
 def test_page_size_one(fmha, orc):
     """A page list with one token per page (the layout some serving stacks use): prefill and decode."""
     w = gen.workload_varlen_prefill(seed=74, batch=4, hq=4, hk=2, head_dim=128, min_len=3, max_len=300, page_size=1)

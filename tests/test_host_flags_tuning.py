@@ -152,3 +152,29 @@ def test_tune_num_splits_picks_the_fastest_and_respects_existing_records(tmp_pat
     assert tuning.tune_num_splits(ran.append, timer, [1, 2], "p", cache=c)["num_splits"] == 2 and ran == [1, 2]
     with pytest.raises(ValueError):
         tuning.tune_num_splits(ran.append, timer, [0, 129], "q", cache=c)
+
+
+def test_tuner_records_the_kernel_variant_with_the_split_count(tmp_path):
+    """Pairs (split count, variant) are measured, a pair the problem cannot take is skipped, and the record carries the
+    winning variant and the kernel that ran; choose_splitkv hands both back."""
+    c = tuning.TuningCache(str(tmp_path), ENV)
+    cost = {(2, 1): 4e-4, (2, 2): 3e-4, (4, 1): 2e-4, (4, 2): None}   # (4, 2) is refused
+    ran = []
+
+    def run(ns, variant):
+        if cost[(ns, variant)] is None:
+            raise ValueError("variant 2 needs an even head count")
+        ran.append((ns, variant))
+        return f"kernel<v{variant}>"
+
+    def timer(fn, cold, repeats):
+        fn()
+        return cost[ran[-1]]
+
+    rec = tuning.tune_num_splits(run, timer, [2, 4], "p2", cache=c, variants=(1, 2))
+    assert (rec["num_splits"], rec["variant"], rec["kernel"]) == (4, 1, "kernel<v1>")
+    assert set(rec["tried_us"]) == {"2/v1", "2/v2", "4/v1"}
+    args = (4, 16, 4, 1, 2048, 128, 64, "bf16")
+    c.insert(tuning.SPLITKV, tuning.splitkv_problem(*args), rec)
+    assert tuning.choose_splitkv(lambda: 7, *args, cache=c) == (4, 1)
+    assert tuning.choose_splitkv(lambda: 7, 8, 16, 4, 1, 2048, 128, 64, "bf16", cache=c) == (7, 0)   # another class: heuristic
