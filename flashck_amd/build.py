@@ -59,7 +59,26 @@ def build(verbose=False, extra_flags=()):
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}")
     os.replace(tmp, LIB)
+    build_header_test()
     return LIB
+
+
+def build_header_test():
+    """tests/cpp/fmha_header_gpu: the C++ program the GPU test of the header API (include/flashck/fmha/fmha_fwd.h)
+    runs.  Built here, next to the library it links, so that it exists wherever the library does; skipped when the
+    test sources are not part of the tree."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "cpp", "fmha_header_gpu.cpp")
+    if not os.path.exists(src):
+        return None
+    exe = src[:-len(".cpp")]
+    cmd = [hipcc(), "-std=c++17", "-O1", "-Wall", "-I", os.path.join(root, "include"), src, "-o", exe + ".tmp", "-L", HERE,
+           "-lflashck_fmha", "-Wl,-rpath,$ORIGIN/../../flashck_amd"]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building {exe} failed:\n{r.stdout}")
+    os.replace(exe + ".tmp", exe)
+    return exe
 
 
 if __name__ == "__main__":
