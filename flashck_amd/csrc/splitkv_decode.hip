@@ -195,10 +195,10 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
     // one lane's piece of a K/V row: 8 elements, as they come from memory and as they go to LDS
     auto fetch = [](const kv_elem* p) -> u32x4_t {
         if constexpr (kKv8) {
-            const u32x2_t v = *reinterpret_cast<const u32x2_t*>(p);
+            const u32x2_t v = ldg8_stream(p);
             return u32x4_t{v[0], v[1], 0u, 0u};
         } else {
-            return ldg16(p);
+            return ldg16_stream(p);
         }
     };
     auto staged = [](u32x4_t v) -> u32x4_t {
