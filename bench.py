@@ -122,6 +122,8 @@ def bench_decode(args, torch, fmha, gen, which):
         else:
             ns = args.paged_splits or fmha.num_splits_heuristic(32, 32, 8, 1, max(w["lens"]), 128)
             name = f"paged-KV decode: B=32 q=1 Hq32/Hk8 D128 L~U[512,4096] P=128 ns={ns} + combine (bf16)"
+            if getattr(args, "paged_variant", 0):
+                name += f" [kernel variant {args.paged_variant}]"
     B, _, Hq, D = w["q"].shape
     Hk = w["k_cache"].shape[2]
     dev = "cuda"
@@ -142,6 +144,7 @@ def bench_decode(args, torch, fmha, gen, which):
     o = torch.empty(B, 1, Hq, D, dtype=q.dtype, device=dev)
 
     fused = getattr(args, "decode_path", "two-launch") == "fused"
+    variant = getattr(args, "paged_variant", 0) if which == "paged_decode" else 0
 
     def step(i, ev):
         kc, vc = pools[i % len(pools)]
@@ -150,7 +153,8 @@ def bench_decode(args, torch, fmha, gen, which):
         if fused:
             fmha.fmha_fwd_splitkv_fused(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], out=o)
         else:
-            fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc, **scales)
+            fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc,
+                                  decode_variant=variant, **scales)
         if ev is not None:
             ev[1].record()
         if not fused:
@@ -298,6 +302,23 @@ def main():
             return dict(workload=r2["name"], us_per_call=r2["ms_per_step"] * 1e3, gbs=r2["gbs"],
                         pct_of_hbm_peak=100 * r2["gbs"] / HBM_PEAK_GBS, kernel_us=r2["kernel_ms"] * 1e3, bytes=r2["bytes"])
 
+        def paged_tuned():
+            # the library's tuning flow on this workload: measure (split count, kernel variant) pairs, run the winner
+            import tempfile
+            from flashck_amd.utils import tuning
+            w = gen.workload_paged_decode()
+            t = [w[k].to("cuda") for k in ("q", "k_cache", "v_cache", "seqlen_k", "block_table")]
+            with tempfile.TemporaryDirectory() as tmp:
+                rec = fmha.tune_decode_num_splits(*t, max_seqlen_k=max(w["lens"]), candidates=(1, 2, 3, 4, 6, 8), variants=(1, 2),
+                                                  cache=tuning.TuningCache(directory=tmp), scale=w["scale"])
+            del t
+            a2 = argparse.Namespace(**vars(args))
+            a2.steps, a2.warmup, a2.paged_splits, a2.paged_variant = max(20, args.steps // 2), 10, rec["num_splits"], rec["variant"]
+            r2 = bench_decode(a2, torch, fmha, gen, "paged_decode")
+            return dict(workload=r2["name"], us_per_call=r2["ms_per_step"] * 1e3, gbs=r2["gbs"],
+                        pct_of_hbm_peak=100 * r2["gbs"] / HBM_PEAK_GBS, kernel_us=r2["kernel_ms"] * 1e3, kernel=r2["kernel"],
+                        num_splits=rec["num_splits"], variant=rec["variant"], tried_us=rec["tried_us"])
+
         def append():
             r4 = bench_appendkv(args, torch, fmha, gen, 100, 10)
             return dict(workload=r4["name"], us_per_call=r4["us_per_call"], bytes=r4["bytes"], new_tokens=r4["new_tokens"])
@@ -321,6 +342,7 @@ def main():
         secondary("splitkv_fused", lambda: splitkv_variant("fused", 0))
         secondary("splitkv_fp8_cache", lambda: splitkv_variant("two-launch", ns_lib, kv_fp8=True))
         secondary("paged_decode", paged)
+        secondary("paged_decode_tuned", paged_tuned)
         secondary("appendkv", append)
         for d in (128, 256):
             secondary(f"prefill_d{d}", lambda d=d: prefill(d))

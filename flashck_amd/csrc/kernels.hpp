@@ -48,6 +48,7 @@ struct SplitKvArgs {
     int32_t variant;   // 0: chosen by the launcher; 1: one KV head per workgroup; 2: head pairs
     int32_t kv8;       // K and V are fp8 (e4m3); the K scale is folded into scale_log2 / mod.scale by the caller
     float v_descale;   // factor on the output (1 unless V is quantised)
+    int32_t longest_first;  // set by the launcher: workgroups take the sequences in order of decreasing key count
 };
 
 struct CombineArgs {

@@ -599,11 +599,12 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
 
 
 def tune_decode_num_splits(q, k_cache, v_cache, seqlen_k, block_table, *, max_seqlen_k: int,
-                           candidates=(1, 2, 4, 8, 16, 32, 64), variants=(0,), **kwargs) -> dict:
+                           candidates=(1, 2, 4, 8, 16, 32, 64), variants=(0,), cache=None, **kwargs) -> dict:
     """Time `fmha_decode_paged` with each candidate (split count, kernel variant) on these tensors and record the
     fastest for the problem class (see utils/tuning.py); later calls with num_splits = 0 on problems of that class use
     both.  variants: 0 = the library's own choice, 1 = one KV head per workgroup, 2 = head pairs (skipped where the
-    problem cannot take it).  Returns the record ({"num_splits", "variant", "kernel", "latency_us", "tried_us", ...})."""
+    problem cannot take it).  cache: the tuning.TuningCache to record into (default: the process-wide one).  Returns
+    the record ({"num_splits", "variant", "kernel", "latency_us", "tried_us", ...})."""
     Hq, D = q.shape[-2], q.shape[-1]
     Hk, page = k_cache.shape[2], k_cache.shape[1]
     B = seqlen_k.numel()
@@ -619,7 +620,7 @@ def tune_decode_num_splits(q, k_cache, v_cache, seqlen_k, block_table, *, max_se
                           workspace=ws[ns], decode_variant=variant, **kwargs)
         return _lib.load().fck_fmha_last_kernel().decode()
 
-    return tuning.tune_num_splits(run, tuning.gpu_timer, candidates, problem, variants=variants)
+    return tuning.tune_num_splits(run, tuning.gpu_timer, candidates, problem, cache=cache, variants=variants)
 
 
 class DecodeWorkspace:

@@ -129,6 +129,28 @@ def test_batch_cache_with_cache_batch_idx(fmha, orc):
     assert_close(o, ro, 1e-2, "o")
 
 
+@pytest.mark.parametrize("variant,num_splits,batch", [(1, 1, 48), (1, 2, 30), (2, 3, 30), (1, 1, 64)])
+def test_ragged_batch_taken_longest_first(fmha, orc, variant, num_splits, batch):
+    # between one and two workgroups per CU the kernel deals its workgroup ids to the sequences in order of decreasing
+    # length (equal lengths: in index order); every sequence must still come out in its own place
+    g = torch.Generator().manual_seed(41 + batch)
+    lens = gen.randint_list(1, 300, batch, g)
+    lens[3] = lens[7] = lens[11] = max(lens)  # ties, also for the first place
+    lens[5] = lens[6] = 1
+    kv = gen.paged_kv(lens, 8, 128, torch.bfloat16, g, 64)
+    kv["q"] = gen.randn((batch, 1, 32, 128), torch.bfloat16, g)
+    scale = 1 / math.sqrt(128)
+    args = dict(seqlen_k=dev(kv["seqlen_k"]), block_table=dev(kv["block_table"]), scale=scale)
+    o_acc, lse_acc = fmha.fmha_fwd_splitkv(dev(kv["q"]), dev(kv["k_cache"]), dev(kv["v_cache"]), num_splits, decode_variant=variant, **args)
+    o = fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, torch.bfloat16)
+    torch.cuda.synchronize()
+    kw = dict(seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], scale=scale)
+    ro_acc, rlse_acc = orc.fmha_splitkv(kv["q"], kv["k_cache"], kv["v_cache"], num_splits, **kw)
+    assert_lse_close(lse_acc, rlse_acc, what="lse_acc")
+    assert_close(o_acc, ro_acc, ATOL[torch.bfloat16], "o_acc")
+    assert_close(o, orc.fmha_fwd(kv["q"], kv["k_cache"], kv["v_cache"], **kw), ATOL[torch.bfloat16], "o")
+
+
 def test_workload2_full(fmha, orc):
     w = gen.workload_paged_decode()
     ns = fmha.num_splits_heuristic(32, 32, 8, 1, max(w["lens"]), 128)
