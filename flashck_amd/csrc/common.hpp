@@ -161,7 +161,8 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 constexpr int kCombineBatch = 16;
 
 template <int DV>
-__device__ __forceinline__ f32x4_t combine_splits(const float* lse_acc, const float* o_acc, int64_t w0, int64_t step, int ns, int c)
+__device__ __forceinline__ f32x4_t combine_splits(const float* lse_acc, const float* o_acc, int64_t w0, int64_t step, int ns, int c,
+                                                  int dv = DV)  // dv: floats per partial row as stored (<= DV)
 {
     float m_run = -INFINITY, sum = 0.f;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -174,7 +175,7 @@ __device__ __forceinline__ f32x4_t combine_splits(const float* lse_acc, const fl
             const int64_t w = w0 + (ok ? s0 + j : s0) * step;  // out-of-range slots re-read a valid one and are dropped
             const float lj = lse_acc[w];
             l[j] = ok ? lj : -INFINITY;
-            v[j] = *reinterpret_cast<const f32x4_t*>(o_acc + w * DV + c);
+            v[j] = *reinterpret_cast<const f32x4_t*>(o_acc + w * dv + c);
         }
         float mb = l[0];
 #pragma unroll

@@ -33,9 +33,19 @@ int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, i
         return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
     if (batch <= 0 || hq <= 0 || hk <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch and head counts must be positive");
     if (hq % hk != 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_num_heads %ld is not a multiple of kv_num_heads %ld", (long)hq, (long)hk);
-    if (d != dv) return fail(FCK_ERR_UNSUPPORTED, "qk_head_dim %ld != v_head_dim %ld is not supported", (long)d, (long)dv);
-    if (d != 64 && d != 128 && d != 256) return fail(FCK_ERR_UNSUPPORTED, "head_dim %ld: kernels exist for 64, 128, 256", (long)d);
+    // Kernels are built for head dims 64, 128 and 256; any other qk_head_dim / v_head_dim (the two may differ) that is a
+    // multiple of 8 runs on the next larger one with the missing columns read as zeros (the reference's
+    // is_pad_qk_head_dim / is_pad_v_head_dim traits, fmha_fwd_split_kv_codegen.h:106-107).
+    if (d < 8 || dv < 8 || d > 256 || dv > 256 || d % 8 || dv % 8)
+        return fail(FCK_ERR_UNSUPPORTED, "qk_head_dim %ld / v_head_dim %ld: head dims are multiples of 8 in [8, 256]", (long)d, (long)dv);
     return FCK_OK;
+}
+
+// head dim the kernels are instantiated for
+int kernel_dim(int64_t d, int64_t dv)
+{
+    const int64_t m = d > dv ? d : dv;
+    return m <= 64 ? 64 : m <= 128 ? 128 : 256;
 }
 
 // Bias / ALiBi / soft cap of a call: `bias` is the positional pointer of the entry points that have one (else null).
@@ -49,6 +59,7 @@ int no_kv_dtype(const fck_fmha_attrs* at)
 int fill_mod(fck::ScoreMod& m, const void* bias, const fck_fmha_attrs* at, float scale, uint32_t mask_type, int64_t hq)
 {
     m = fck::ScoreMod{};
+    m.scale = scale;
     if (!at) {
         if (bias) return fail(FCK_ERR_UNSUPPORTED, "a bias pointer needs the _attrs entry point: fck_fmha_attrs says what it holds");
         return FCK_OK;
@@ -193,6 +204,9 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
     a.hk = (int32_t)hk;
     a.num_splits = (int32_t)num_splits;
     a.shape_sq = seqlen_q;  // group mode: seqlen_q carries total_q (the "shape" length of the FlashCK wrapper)
+    a.d = (int32_t)d;
+    a.dv = (int32_t)dv;
+    const bool padded = d != dv || d != kernel_dim(d, dv);
     a.scale_log2 = scale * fck::kLog2e;
     a.mask_type = mask_type;
     a.window_left = window_left;
@@ -202,9 +216,9 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
     if (attrs && attrs->decode_variant != 0) {
         if (attrs->decode_variant != 1 && attrs->decode_variant != 2)
             return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant %d out of range [0,2]", attrs->decode_variant);
-        if (attrs->decode_variant == 2 && (hk % 2 || d > 128 || q_max_seq_len * (hq / hk) > 16 || a.mod.active()))
-            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant 2 (head pairs) needs an even kv_num_heads, head dim <= 128, at most 16 packed "
-                                                  "query rows and no bias / soft cap");
+        if (attrs->decode_variant == 2 && (hk % 2 || d > 128 || padded || q_max_seq_len * (hq / hk) > 16 || a.mod.active()))
+            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant 2 (head pairs) needs an even kv_num_heads, head dim 64 or 128, at most 16 "
+                                                  "packed query rows and no bias / soft cap");
         a.variant = attrs->decode_variant;
     }
     if (attrs && attrs->kv_dtype != 0) {
@@ -214,6 +228,7 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
         if (!(kd > 0.f) || !std::isfinite(kd) || !(vd > 0.f) || !std::isfinite(vd))
             return fail(FCK_ERR_INVALID_ARGUMENT, "k_descale and v_descale must be positive and finite (0: 1)");
         if (!aligned16(k) || !aligned16(v)) return fail(FCK_ERR_INVALID_ARGUMENT, "k and v must be 16-byte aligned");
+        if (padded) return fail(FCK_ERR_UNSUPPORTED, "an fp8 K/V cache needs qk_head_dim = v_head_dim in {64, 128, 256}");
         a.kv8 = 1;
         a.scale_log2 *= kd;
         a.mod.scale *= kd;
@@ -286,7 +301,8 @@ int fck_fmha_fwd_splitkv_attrs(const void* q, const void* k, const void* v, cons
         "splitkv_decode_kernel<row_lookup,kv_fp8>",  "splitkv_decode_kernel<uniform_page,kv_fp8>",
         "splitkv_decode_kernel<row_lookup,kv_fp8,score_mod>", "splitkv_decode_kernel<uniform_page,kv_fp8,score_mod>"};
     g_kernel = names[(a.kv8 ? 4 : 0) + (a.mod.active() ? 2 : 0) + (uniform ? 1 : 0)];
-    return launch_status(fck::launch_splitkv_decode(a, (int)d, dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
+    if (d != dv || d != kernel_dim(d, dv)) g_kernel = uniform ? "splitkv_decode_kernel<uniform_page,padded_head_dim>" : "splitkv_decode_kernel<row_lookup,padded_head_dim>";
+    return launch_status(fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
                          "FmhaFwdSplitKV launch");
 }
 
@@ -314,10 +330,12 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
         return rc;
     if (!o) return fail(FCK_ERR_INVALID_ARGUMENT, "o must not be null");
     if (!aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "o must be 16-byte aligned");
+    if (d != dv || d != kernel_dim(d, dv))
+        return fail(FCK_ERR_UNSUPPORTED, "the fused split-KV entry point needs qk_head_dim = v_head_dim in {64, 128, 256}");
     // The partial results and the arrival tickets live in a fixed device array of the library: nothing is allocated.
     const int64_t shape_batch = seqstart_q ? 1 : batch;
     const int64_t part_rows = shape_batch * hq * num_splits * seqlen_q;
-    const int64_t m_tiles = fck::splitkv_decode_m_tiles((int)d, rows_max);
+    const int64_t m_tiles = fck::splitkv_decode_m_tiles(kernel_dim(d, dv), rows_max);
     const int64_t tickets = batch * hk * m_tiles;
     if (part_rows * (dv + 1) > fck::kDecodeScratchPartialFloats || tickets > fck::kDecodeScratchTickets)
         return fail(FCK_ERR_UNSUPPORTED,
@@ -332,7 +350,7 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
     a.lse_acc = a.o_acc + part_rows * dv;
     a.o = o;
     g_kernel = uniform ? "splitkv_decode_kernel<uniform_page,fused>" : "splitkv_decode_kernel<row_lookup,fused>";
-    return launch_status(fck::launch_splitkv_decode(a, (int)d, dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
+    return launch_status(fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
                          "FmhaFwdSplitKV (fused) launch");
 }
 
@@ -346,7 +364,7 @@ int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o
         return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
     if (!lse_acc || !o_acc || !o) return fail(FCK_ERR_INVALID_ARGUMENT, "lse_acc, o_acc and o must not be null");
     if (batch <= 0 || hq <= 0 || seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch, q_num_heads and seqlen_q must be positive");
-    if (dv != 64 && dv != 128 && dv != 256) return fail(FCK_ERR_UNSUPPORTED, "v_head_dim %ld: kernels exist for 64, 128, 256", (long)dv);
+    if (dv < 8 || dv > 256 || dv % 8) return fail(FCK_ERR_UNSUPPORTED, "v_head_dim %ld: a multiple of 8 in [8, 256]", (long)dv);
     if (num_splits < 1 || num_splits > 128) return fail(FCK_ERR_INVALID_ARGUMENT, "num_splits %ld out of range [1,128]", (long)num_splits);
     if (!aligned16(o_acc) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_acc and o must be 16-byte aligned");
     fck::CombineArgs a{};
@@ -415,10 +433,13 @@ int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* kne
     return launch_status(fck::launch_appendkv(a, dtype, (int)seqlen_knew, static_cast<hipStream_t>(stream)), "FmhaFwdAppendKV launch");
 }
 
-static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t q_max_seq_len, bool uniform, void* stream,
+static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t dtype, int64_t q_max_seq_len, bool uniform, void* stream,
                           const char* what)
 {
     if (q_max_seq_len <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_max_seq_len must be positive");
+    a.d = (int32_t)d_qk;
+    a.dv = (int32_t)dv;
+    const int64_t d = kernel_dim(d_qk, dv);
     // The direct-to-LDS kernels address a tile's rows with 32-bit byte offsets from the tile's first row.
     if ((int64_t)a.hk * d * 2 * 64 >= ((int64_t)1 << 31))
         return fail(FCK_ERR_INVALID_ARGUMENT, "kv_num_heads * head_dim = %ld is too large (64 cache rows must span < 2 GiB)", (long)(a.hk * d));
@@ -426,6 +447,12 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d, int32_t dtype, int64_t
     // takes the 4-wave kernel that sends K/V tiles straight to LDS (128 rows per workgroup) when a 64-key tile never
     // straddles a page; short runs at head dim <= 128 and page sizes that are not a multiple of 64 take the 4-wave
     // kernel that stages K/V through registers.
+    if (d_qk != d || dv != d) {
+        // head dims other than 64 / 128 / 256, or qk_head_dim != v_head_dim: the register-staged kernel pads them
+        a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
+        g_kernel = uniform ? "prefill_kernel<uniform_page,padded_head_dim>" : "prefill_kernel<row_lookup,padded_head_dim>";
+        return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+    }
     if (a.mod.active()) {
         // bias, ALiBi and the soft cap are applied by the register-staged kernel only
         a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
@@ -494,7 +521,7 @@ int fck_fmha_fwd_attrs(const void* q, const void* k, const void* v, const void* 
         a.kv.seqlen_k = (int32_t)seqlen_k;
         if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
     }
-    return prefill_common(a, d, dtype, q_max_seq_len, true, stream, "FmhaFwd launch");
+    return prefill_common(a, d, dv, dtype, q_max_seq_len, true, stream, "FmhaFwd launch");
 }
 
 int fck_fmha_batch_prefill(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
@@ -545,7 +572,7 @@ int fck_fmha_batch_prefill_attrs(const void* q, const void* k_cache, const void*
     a.kv.page_shift = log2_exact(page_block_size);
     if (num_total_pages * page_block_size > INT32_MAX)
         return fail(FCK_ERR_INVALID_ARGUMENT, "a pool of %ld x %ld cache rows exceeds the 2^31 - 1 rows the kernels index", (long)num_total_pages, (long)page_block_size);
-    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdBatchPrefill launch");
+    return prefill_common(a, d, dv, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdBatchPrefill launch");
 }
 
 int fck_fmha_fwd_pagedkv(const void* q, const void* k_cache, const void* v_cache, void* o, const int32_t* seqstart_q,
@@ -597,7 +624,7 @@ int fck_fmha_fwd_pagedkv_attrs(const void* q, const void* k_cache, const void* v
     a.kv.page_size = (int32_t)page_block_size;
     a.kv.page_shift = log2_exact(page_block_size);
     if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
-    return prefill_common(a, d, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdPagedKV launch");
+    return prefill_common(a, d, dv, dtype, q_max_seq_len, page_block_size % 64 == 0, stream, "FmhaFwdPagedKV launch");
 }
 
 }  // extern "C"

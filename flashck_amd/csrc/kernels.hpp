@@ -49,6 +49,7 @@ struct SplitKvArgs {
     int32_t kv8;       // K and V are fp8 (e4m3); the K scale is folded into scale_log2 / mod.scale by the caller
     float v_descale;   // factor on the output (1 unless V is quantised)
     int32_t longest_first;  // set by the launcher: workgroups take the sequences in order of decreasing key count
+    int32_t d, dv;     // head dims of Q/K and of V/O as stored (multiples of 8); the kernel's D is the next of 64 / 128 / 256
 };
 
 struct CombineArgs {
@@ -92,6 +93,7 @@ struct PrefillArgs {
     uint32_t mask_type;
     int64_t window_left, window_right;
     ScoreMod mod;  // bias / ALiBi / soft cap; all zero: none (only the 4-wave kernel of prefill.hip applies them)
+    int32_t d, dv;  // head dims of Q/K and of V/O as stored; other than the kernel's D only in the 4-wave kernel of prefill.hip
 };
 
 hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page, int num_cu,

@@ -33,9 +33,14 @@ constexpr size_t prefill_lds_bytes()
     return (size_t)4 * PrefillShape<D>::TILEB;
 }
 
-template <typename T, int D, bool kUniformPage, bool kMod = false>
+// kPad: the stored head dims (a.d for Q/K, a.dv for V/O; multiples of 8) are smaller than D.  Rows are a.d / a.dv
+// elements apart and the 16-byte pieces past a row's end are zeros instead of loads: zero columns of Q and K add
+// nothing to a score, zero columns of V give output columns that are not stored.
+template <typename T, int D, bool kUniformPage, bool kMod = false, bool kPad = false>
 __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const PrefillArgs a)
 {
+    const int dq = kPad ? a.d : D;    // elements per stored Q / K row
+    const int dvs = kPad ? a.dv : D;  // elements per stored V / O row
     typedef PrefillShape<D> S;
     typedef typename T::vec8 vec8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -92,12 +97,12 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
     // ---- Q fragments (B operand of S^T = K . Q^T): lane (row = l32, k-group = half) ------------------------------
     vec8 qf[S::KT];
     {
-        const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * D +
+        const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * dq +
                              half * 8;
 #pragma unroll
         for (int t = 0; t < S::KT; ++t) {
             u32x4_t v = {0u, 0u, 0u, 0u};
-            if (row_ok) v = ldg16(qp + t * 16);
+            if (row_ok && (!kPad || t * 16 + half * 8 < dq)) v = ldg16(qp + t * 16);
             qf[t] = as_vec8<vec8>(v);
         }
     }
@@ -111,8 +116,14 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
 
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k);
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v);
-    const int64_t row_stride = (int64_t)a.hk * D;
     const int last_key = sk_b - 1;
+    // this thread's piece u of a K / V row: offset inside the row's cache line-up, or zeros when the row ends before it
+    auto load_piece = [&](const uint16_t* base, int64_t row, int c, int dim) -> u32x4_t {
+        if constexpr (kPad) {
+            if (c * 8 >= dim) return u32x4_t{0u, 0u, 0u, 0u};
+        }
+        return ldg16(base + (row * a.hk + hkv) * dim + c * 8);
+    };
 
     // global -> LDS copy assignment: 16-byte chunk (row, c) per thread and step
     int cp_row[S::LD], cp_c[S::LD], cp_koff[S::LD], cp_voff[S::LD];
@@ -134,17 +145,17 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
             const int room = last_key - kb;
 #pragma unroll
             for (int u = 0; u < S::LD; ++u) {
-                const int64_t off = (row0 + min(cp_row[u], room)) * row_stride + hkv * D + cp_c[u] * 8;
-                kreg[u] = ldg16(kp + off);
-                vreg[u] = ldg16(vp + off);
+                const int64_t row = row0 + min(cp_row[u], room);
+                kreg[u] = load_piece(kp, row, cp_c[u], dq);
+                vreg[u] = load_piece(vp, row, cp_c[u], dvs);
             }
         } else {
 #pragma unroll
             for (int u = 0; u < S::LD; ++u) {
                 const int key = min(kb + cp_row[u], last_key);
-                const int64_t off = kv_row(a.kv, ks, key) * row_stride + hkv * D + cp_c[u] * 8;
-                kreg[u] = ldg16(kp + off);
-                vreg[u] = ldg16(vp + off);
+                const int64_t row = kv_row(a.kv, ks, key);
+                kreg[u] = load_piece(kp, row, cp_c[u], dq);
+                vreg[u] = load_piece(vp, row, cp_c[u], dvs);
             }
         }
     };
@@ -279,11 +290,14 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
     l_run = pair32_sum(l_run);
     if (row_ok) {
         const float inv = (l_run == 0.f) ? 0.f : 1.f / l_run;
-        uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * D;
+        uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * dvs;
 #pragma unroll
         for (int dvb = 0; dvb < S::DVB; ++dvb)
 #pragma unroll
             for (int j4 = 0; j4 < 4; ++j4) {
+                if constexpr (kPad) {
+                    if (dvb * 32 + j4 * 8 + half * 4 >= dvs) continue;
+                }
                 u32x2_t out;
                 out[0] = T::pack2(oacc[dvb][j4 * 4 + 0] * inv, oacc[dvb][j4 * 4 + 1] * inv);
                 out[1] = T::pack2(oacc[dvb][j4 * 4 + 2] * inv, oacc[dvb][j4 * 4 + 3] * inv);
@@ -297,6 +311,10 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
 {
     const dim3 grid(a.m_tiles, a.hq, a.batch);
     constexpr size_t lds = prefill_lds_bytes<D>();
+    if (a.d != D || a.dv != D) {  // padded head dims: the general kernel (modifiers on, identity when there are none)
+        if (uniform) return launch_with_lds<prefill_kernel<T, D, true, true, true>>(grid, dim3(256), lds, st, a);
+        return launch_with_lds<prefill_kernel<T, D, false, true, true>>(grid, dim3(256), lds, st, a);
+    }
     if (a.mod.active()) {
         if (uniform) return launch_with_lds<prefill_kernel<T, D, true, true>>(grid, dim3(256), lds, st, a);
         return launch_with_lds<prefill_kernel<T, D, false, true>>(grid, dim3(256), lds, st, a);

@@ -1,7 +1,8 @@
 // LSE combine of split-KV partial results (gfx950).
 //   LSE = logsumexp_s lse_acc[s];  O = sum_s exp(lse_acc[s] - LSE) * o_acc[s]  -> T
 // A pure streaming reduce: DV/4 lanes own one output row with float4 loads of each split's partial row.
-// Layouts: o_acc [Bs, Hq, ns, Sq, Dv], lse_acc [Bs, Hq, ns, Sq], o [Bs*Sq, Hq, Dv].
+// Layouts: o_acc [Bs, Hq, ns, Sq, Dv], lse_acc [Bs, Hq, ns, Sq], o [Bs*Sq, Hq, Dv].  Dv is any multiple of 8 up to 256: the
+// kernel is instantiated for DV = 64 / 128 / 256 and the lanes past Dv of a row's group idle.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -14,18 +15,18 @@ __global__ __launch_bounds__(256) void splitkv_combine_kernel(const CombineArgs 
     constexpr int RPB = 256 / TPR;  // rows per block
     const int64_t item = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;  // (row, head) pair
     const int c = (threadIdx.x % TPR) * 4;
-    if (item >= a.rows * a.hq) return;
+    if (item >= a.rows * a.hq || c >= a.dv) return;
     const int64_t row = item / a.hq;  // b * Sq + i
     const int h = (int)(item % a.hq);
     const int64_t b = row / a.Sq, i = row % a.Sq;
     const int ns = a.num_splits;
     const int64_t w0 = ((b * a.hq + h) * ns) * a.Sq + i;  // split 0; next split is Sq further
 
-    const f32x4_t acc = combine_splits<DV>(a.lse_acc, a.o_acc, w0, a.Sq, ns, c);
+    const f32x4_t acc = combine_splits<DV>(a.lse_acc, a.o_acc, w0, a.Sq, ns, c, a.dv);
     u32x2_t out;
     out[0] = T::pack2(acc[0], acc[1]);
     out[1] = T::pack2(acc[2], acc[3]);
-    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.o) + (row * a.hq + h) * DV + c) = out;
+    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.o) + (row * a.hq + h) * a.dv + c) = out;
 }
 
 template <typename T, int DV>
@@ -41,12 +42,10 @@ static hipError_t launch_dv(const CombineArgs& a, hipStream_t st)
 template <typename T>
 static hipError_t launch_t(const CombineArgs& a, hipStream_t st)
 {
-    switch (a.dv) {
-    case 64: return launch_dv<T, 64>(a, st);
-    case 128: return launch_dv<T, 128>(a, st);
-    case 256: return launch_dv<T, 256>(a, st);
-    }
-    return hipErrorInvalidValue;
+    if (a.dv <= 0 || a.dv > 256 || a.dv % 8) return hipErrorInvalidValue;
+    if (a.dv <= 64) return launch_dv<T, 64>(a, st);
+    if (a.dv <= 128) return launch_dv<T, 128>(a, st);
+    return launch_dv<T, 256>(a, st);
 }
 
 hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st)

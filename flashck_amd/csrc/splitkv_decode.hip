@@ -61,10 +61,16 @@ __device__ __forceinline__ int v_swizzle(int key)
 
 // kKv8: K and V are stored as fp8 (e4m3, one byte per element) and widened to T on their way into LDS; everything after
 // the staging tile is the 16-bit path.  A lane then loads 8 bytes where the 16-bit path loads 16.
-template <typename T, int D, int NW, int MB, int HG, bool kUniformPage, bool kMod = false, bool kKv8 = false>
+// kPad: the stored head dims (a.d for Q/K, a.dv for V and the output; multiples of 8) are smaller than D: rows are
+// a.d / a.dv elements apart, and the 16-byte pieces past a row's end are zeros instead of loads (a zero column of Q and K
+// adds nothing to a score, a zero column of V gives an output column that is not stored).
+template <typename T, int D, int NW, int MB, int HG, bool kUniformPage, bool kMod = false, bool kKv8 = false, bool kPad = false>
 __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvArgs a)
 {
     static_assert(!kMod || HG == 1, "score modifiers are per head: one KV head per workgroup");
+    static_assert(!kPad || (HG == 1 && !kKv8), "padded head dims: one KV head per workgroup, 16-bit cache");
+    const int dq = kPad ? a.d : D;   // elements per stored Q / K row
+    const int dvs = kPad ? a.dv : D;  // elements per stored V / partial-output row
     typedef DecodeShape<D, HG> S;
     typedef typename T::vec8 vec8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -180,11 +186,11 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
         for (int hl = 0; hl < HG; ++hl)
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
-                const int64_t off = ((int64_t)(q_row0 + row_i[mb]) * a.hq + (hkv0 + hl) * g + row_hl[mb]) * D + kg * 8;
+                const int64_t off = ((int64_t)(q_row0 + row_i[mb]) * a.hq + (hkv0 + hl) * g + row_hl[mb]) * dq + kg * 8;
 #pragma unroll
                 for (int t = 0; t < S::KT; ++t) {
                     u32x4_t v = {0u, 0u, 0u, 0u};
-                    if (row_ok[mb]) v = ldg16(qp + off + t * 32);
+                    if (row_ok[mb] && (!kPad || t * 32 + kg * 8 < dq)) v = ldg16(qp + off + t * 32);
                     qf[hl][mb][t] = as_vec8<vec8>(v);
                 }
             }
@@ -224,7 +230,6 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
             return v;
         }
     };
-    const int64_t krow_stride = (int64_t)a.hk * D;
     const int last_key = sk_b - 1;
 
     // ---- this wave's staging tiles and its lanes' places in them -----------------------------------------------------
@@ -285,23 +290,37 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
         return ks.base_row + kb;
     };
     // global offset (in elements) of this lane's piece for load instruction u of tile c (first cache row row0)
-    auto src_off = [&](int c, int u, int64_t row0) -> int64_t {
+    // (dim: elements per stored row of the operand, dq for K and dvs for V)
+    auto src_off = [&](int c, int u, int64_t row0, int dim) -> int64_t {
         const int kb = (t_begin + c) * S::TK;
         if constexpr (kUniformPage) {
             // the whole tile lies in one page (or the cache is contiguous): one row base per tile;
             // rows past the last key repeat it (their scores are masked)
             const int kl = min(u * S::KPI + ld_key, last_key - kb);
-            return (row0 + kl) * krow_stride + hkv0 * D + ld_piece * 8;
+            return ((row0 + kl) * a.hk + hkv0) * dim + ld_piece * 8;
         } else {
             const int key = min(kb + u * S::KPI + ld_key, last_key);
-            return kv_row(a.kv, ks, key) * krow_stride + hkv0 * D + ld_piece * 8;
+            return (kv_row(a.kv, ks, key) * a.hk + hkv0) * dim + ld_piece * 8;
         }
+    };
+    const bool k_piece = !kPad || ld_piece * 8 < dq, v_piece = !kPad || ld_piece * 8 < dvs;  // this lane's piece exists
+    auto fetch_k = [&](int c, int u, int64_t row0) -> u32x4_t {
+        if constexpr (kPad) {
+            if (!k_piece) return u32x4_t{0u, 0u, 0u, 0u};
+        }
+        return fetch(kp + src_off(c, u, row0, dq));
+    };
+    auto fetch_v = [&](int c, int u, int64_t row0) -> u32x4_t {
+        if constexpr (kPad) {
+            if (!v_piece) return u32x4_t{0u, 0u, 0u, 0u};
+        }
+        return fetch(vp + src_off(c, u, row0, dvs));
     };
     auto load_tile = [&](int c, int64_t row0, Frag& f) {
 #pragma unroll
-        for (int u = 0; u < S::VN; ++u) f.a[u] = fetch(kp + src_off(c, u, row0));
+        for (int u = 0; u < S::VN; ++u) f.a[u] = fetch_k(c, u, row0);
 #pragma unroll
-        for (int u = 0; u < S::VN; ++u) f.a[S::VN + u] = fetch(vp + src_off(c, u, row0));
+        for (int u = 0; u < S::VN; ++u) f.a[S::VN + u] = fetch_v(c, u, row0);
     };
     auto store_tile = [&](const Frag& f) {
 #pragma unroll
@@ -314,13 +333,13 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
 #pragma unroll
         for (int u = 0; u < S::VN; ++u) {
             *(u32x4_t FCK_LDS*)(kstage + kw_off[u]) = staged(f.a[u]);
-            f.a[u] = fetch(kp + src_off(c_next, u, row0));
+            f.a[u] = fetch_k(c_next, u, row0);
             __builtin_amdgcn_sched_barrier(0);  // keep the store / load pairs interleaved in this order
         }
 #pragma unroll
         for (int u = 0; u < S::VN; ++u) {
             *(u32x4_t FCK_LDS*)(vstage + vw_off[u]) = staged(f.a[S::VN + u]);
-            f.a[S::VN + u] = fetch(vp + src_off(c_next, u, row0));
+            f.a[S::VN + u] = fetch_v(c_next, u, row0);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -475,6 +494,9 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
                 const int rr = e / D, c = e % D;
                 const int r = r_tile0 + mb * 16 + rr;
                 if (r >= R) continue;
+                if constexpr (kPad) {
+                    if (c >= dvs) continue;
+                }
                 float mmax = -INFINITY;
 #pragma unroll
                 for (int w = 0; w < NW; ++w) mmax = fmaxf(mmax, mlbuf[(w * 2 + 0) * 16 + rr]);
@@ -488,7 +510,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
                 }
                 const int i = r / g, h = (hkv0 + hl) * g + r % g;
                 const int64_t wofs = ((int64_t)(wb * a.hq + h) * a.num_splits + split) * Sq + wrow0 + i;
-                o_acc[wofs * D + c] = (L == 0.f) ? 0.f : acc / L * a.v_descale;
+                o_acc[wofs * dvs + c] = (L == 0.f) ? 0.f : acc / L * a.v_descale;
                 if (c == 0) lse_acc[wofs] = (L == 0.f) ? -INFINITY : (mmax + fast_log2(L)) * kLn2;
             }
         }
@@ -562,6 +584,11 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
     const dim3 block(NW * 64);
     constexpr size_t lds = decode_lds_bytes<D, NW, HG>();
     if constexpr (HG == 1) {
+        if (a.d != D || a.dv != D) {  // padded head dims: the general kernel (modifiers on, identity when there are none)
+            if (a.kv8 || a.tickets) return hipErrorInvalidValue;  // refused by the caller
+            if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true, false, true>>(grid, block, lds, st, a);
+            return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true, false, true>>(grid, block, lds, st, a);
+        }
         if (a.mod.active()) {
             if (a.kv8) {
                 if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true, true>>(grid, block, lds, st, a);
@@ -584,7 +611,7 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
 static bool use_head_pairs(const SplitKvArgs& a, int m_tiles, int num_cu)
 {
     if (a.variant != 0) return a.variant == 2;  // validated by the caller
-    if (a.hk % 2 || a.mod.active()) return false;
+    if (a.hk % 2 || a.mod.active() || a.d != a.dv || (a.d != 64 && a.d != 128)) return false;
     return (int64_t)(a.hk / 2) * a.num_splits * m_tiles * a.batch >= num_cu;
 }
 

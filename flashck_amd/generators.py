@@ -68,11 +68,12 @@ def scatter_to_pages(rows: List[torch.Tensor], table: torch.Tensor, pool: int, p
     return cache
 
 
-def paged_kv(lens, hk, d, dtype, g, page_size=128, slack=0.10, capacity=None, shuffle=True):
-    """Random K/V for sequences of the given lengths, stored in a shuffled paged cache with NaN in unused slots."""
+def paged_kv(lens, hk, d, dtype, g, page_size=128, slack=0.10, capacity=None, shuffle=True, dv=None):
+    """Random K/V for sequences of the given lengths, stored in a shuffled paged cache with NaN in unused slots
+    (dv: head dim of V when it differs from K's)."""
     table, pool = paged_layout(lens, page_size, g, slack, capacity, shuffle)
     k_rows = [randn((n, hk, d), dtype, g) for n in lens]
-    v_rows = [randn((n, hk, d), dtype, g) for n in lens]
+    v_rows = [randn((n, hk, dv or d), dtype, g) for n in lens]
     k_cache = scatter_to_pages(k_rows, table, pool, page_size)
     v_cache = scatter_to_pages(v_rows, table, pool, page_size)
     return dict(k_cache=k_cache, v_cache=v_cache, block_table=table, k_rows=k_rows, v_rows=v_rows,

@@ -100,6 +100,8 @@ typedef struct fck_fmha_attrs {
 #define FCK_OK 0
 #define FCK_ERR_INVALID_ARGUMENT (-1) /* null pointer, non-positive size, Hq % Hk != 0 ... */
 #define FCK_ERR_UNSUPPORTED (-2)      /* dtype / head_dim / feature this build has no kernel for */
+/* Head dims: qk_head_dim and v_head_dim are independent multiples of 8 in [8, 256] (the reference pads them with its
+ * is_pad_qk_head_dim / is_pad_v_head_dim traits, core/profiling/attention/fmha_fwd_split_kv/fmha_fwd_split_kv_codegen.h:106-107). */
 #define FCK_ERR_LAUNCH (-3)           /* the HIP runtime refused the launch */
 
 /* Text of the last error raised on the calling thread ("" when none). */

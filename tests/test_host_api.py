@@ -47,8 +47,10 @@ def test_error_codes_without_a_gpu():
     # Hq not a multiple of Hk
     rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 3, 2, 64, 64, 8, 0.125, -1, -1, 0, 4, None)
     assert rc == -1 and b"multiple" in lib.fck_last_error()
-    # unsupported head dim
-    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 80, 80, 8, 0.125, -1, -1, 0, 4, None)
+    # unsupported head dims: not a multiple of 8, beyond 256
+    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 84, 84, 8, 0.125, -1, -1, 0, 4, None)
+    assert rc == -2 and b"head_dim" in lib.fck_last_error()
+    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 264, 8, 0.125, -1, -1, 0, 4, None)
     assert rc == -2 and b"head_dim" in lib.fck_last_error()
     # null pointer
     rc = lib.fck_fmha_fwd(None, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, 4, None)
@@ -68,7 +70,7 @@ def test_error_codes_without_a_gpu():
                                   0.125, -1, -1, 0, 4, None)
     assert rc == -1 and b"key counts" in lib.fck_last_error()
     # combine: bad head dim; appendkv: odd rotary_dim
-    rc = lib.fck_fmha_fwd_splitkv_combine(p, p, p, None, 1, 1, 2, 96, 1, 2, 4, None)
+    rc = lib.fck_fmha_fwd_splitkv_combine(p, p, p, None, 1, 1, 2, 100, 1, 2, 4, None)
     assert rc == -2
     rc = lib.fck_fmha_fwd_appendkv(None, p, p, p, p, p, None, 1, p, p, 31, 2, 1, p, 4, 16, None, 0, 1, 2, 2, 64, 64, 4, None)
     assert rc == -1 and b"rotary_dim" in lib.fck_last_error()

@@ -136,6 +136,23 @@ def test_addressing_modes_are_bit_identical_to_contiguous(orc, mode):
     assert torch.isfinite(got.float()).all(), "NaN sentinels of unused page slots leaked into the result"
 
 
+@pytest.mark.parametrize("d,dv", [(32, 32), (40, 72), (96, 96), (192, 128), (128, 64), (8, 256)])
+def test_unequal_and_odd_head_dims_match_sdpa(orc, d, dv):
+    # qk_head_dim != v_head_dim and head dims off the 64 / 128 / 256 grid: the library routine takes them as they are
+    g = torch.Generator().manual_seed(d + dv)
+    q, k, v = gen.randn((2, 9, 4, d), torch.bfloat16, g), gen.randn((2, 31, 2, d), torch.bfloat16, g), gen.randn((2, 31, 2, dv), torch.bfloat16, g)
+    o, lse = orc.fmha_fwd(q, k, v, return_lse=True, mask_type=2, window=(-1, 0))
+    vis = flash_mask(2, (-1, 0), 9, 31)
+    assert o.shape == (2, 9, 4, dv)
+    assert (o.float() - sdpa(q, k, v, mask=vis)).abs().max() <= 1.6e-2
+    s = torch.einsum("bqhd,bkhd->bhqk", q.float(), k.float().repeat_interleave(2, 2)) / math.sqrt(d)
+    assert (lse - torch.logsumexp(s.masked_fill(~vis, float("-inf")), -1)).abs().max() <= 1e-4
+    o_acc, lse_acc = orc.fmha_splitkv(q, k, v, 3, mask_type=2, window=(-1, 0))
+    assert o_acc.shape == (2, 4, 3, 9, dv)
+    comb = orc.splitkv_combine(lse_acc, o_acc, torch.bfloat16)
+    assert (comb.float() - o.float()).abs().max() <= 8e-3
+
+
 @pytest.mark.parametrize("ns", [1, 2, 3, 8, 16])
 @pytest.mark.parametrize("mask_type", [0, 2])
 def test_splitkv_partials_and_combine(orc, ns, mask_type):
