@@ -14,6 +14,7 @@
 // otherwise); the first rows of the first kPrefillPageCache key tiles are cached, later tiles are looked up one by one.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "lds_tiles.hpp"
 
 #include <type_traits>
 
@@ -32,10 +33,9 @@ struct Shape {
     static_assert(D >= 128, "swizzles below are those of rows of at least 256 bytes");
 };
 
-// XOR swizzles of the 16-byte chunk index: K is read by 16 consecutive lanes = consecutive rows at one logical chunk,
-// V (transposing read) by 16 lanes = 4 rows x 4 adjacent chunks.
-__device__ __forceinline__ int k_swz(int row) { return row & 15; }
-__device__ __forceinline__ int v_swz(int row, int lc) { return ((row & 3) << 1) ^ (((lc >> 1) & 1) << 3); }
+// swizzles of rows of at least 256 bytes (see lds_tiles.hpp)
+__device__ __forceinline__ int k_swz(int row) { return tiles::k_swz<256>(row); }
+__device__ __forceinline__ int v_swz(int row, int lc) { return tiles::v_swz<256>(row, lc); }
 
 template <typename T, int D>
 __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a)
@@ -136,39 +136,15 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     const int cp_pc = lane & 31;
     const int cp_kc0 = (cp_pc ^ k_swz(cp_row0)) * 8;      // K chunk (element offset in the row), even u
     const int cp_kc1 = (cp_pc ^ k_swz(cp_row0 + 8)) * 8;  // odd u
-    const int cp_t = cp_pc ^ ((cp_row0 & 3) << 1);
-    const int cp_vc = (cp_t ^ (((cp_t >> 1) & 1) << 3)) * 8;  // V chunk: inverse of lc -> lc ^ v_swz(row, lc)
+    const int cp_vc = tiles::v_chunk_at<256>(cp_row0, cp_pc) * 8;  // V chunk
     const uint32_t cp_koff0 = (uint32_t)(cp_row0 * (int)row_stride + cp_kc0) * 2u;  // bytes from row 8u of the tile
     const uint32_t cp_koff1 = (uint32_t)(cp_row0 * (int)row_stride + cp_kc1) * 2u;
     const uint32_t cp_voff = (uint32_t)(cp_row0 * (int)row_stride + cp_vc) * 2u;
 
-    // first cache row of every tile of this workgroup
-    if (ks.table != nullptr) {
-        for (int i = tid; i < min(n, kPrefillPageCache); i += 256) {
-            const int kb = (t_begin + i) * BN;
-            const int pi = a.kv.page_shift >= 0 ? kb >> a.kv.page_shift : kb / a.kv.page_size;
-            row_lds[i] = ks.table[pi] * a.kv.page_size + (kb - pi * a.kv.page_size);
-        }
-    }
-    int row_vec = 0, row_chunk = -1;  // lane l: first row of tile row_chunk * 64 + l
-    auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t {
-        if (ks.table != nullptr) {
-            if (i >= kPrefillPageCache) {
-                // more key tiles than the cache holds (> kPrefillPageCache * 64 keys): one scalar table lookup per tile
-                const int kb = (t_begin + i) * BN;
-                const int pi = a.kv.page_shift >= 0 ? kb >> a.kv.page_shift : kb / a.kv.page_size;
-                int page = ((const __attribute__((address_space(4))) int32_t*)ks.table)[pi];
-                asm volatile("" : "+s"(page));
-                return (int64_t)page * a.kv.page_size + (kb - pi * a.kv.page_size);
-            }
-            if ((i >> 6) != row_chunk) {
-                row_chunk = i >> 6;
-                row_vec = row_lds[min(row_chunk * 64 + lane, kPrefillPageCache - 1)];
-            }
-            return __builtin_amdgcn_readlane(row_vec, i & 63);
-        }
-        return ks.base_row + (t_begin + i) * BN;
-    };
+    // first cache row of every tile of this workgroup (see tiles::FirstRows)
+    tiles::FirstRows<BN> first_rows{row_lds};
+    first_rows.fill(a.kv, ks, t_begin, n, tid, 256);
+    auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t { return first_rows.row0(a.kv, ks, t_begin, i, lane); };
     // request this wave's share of the K and V tile i (local index) into buffer buf
     auto request = [&](int i, int buf) __attribute__((always_inline)) {
         const int room = sk_b - 1 - (t_begin + i) * BN;
@@ -189,20 +165,12 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
                     const int row = min(cp_row0 + 8 * u, room);
                     off = (uint32_t)(row * (int)row_stride + (kv == 0 ? ((u & 1) ? cp_kc1 : cp_kc0) : cp_vc)) * 2u;
                 }
-                // Written as assembly on purpose: a load the compiler knows about makes it drain the whole load queue
-                // before the next LDS read it cannot prove disjoint.  m0 carries the LDS address of the block and is put
-                // back afterwards, since the compiler does not expect it to change.
-                uint32_t m0_saved;
-                const uint32_t dst = (uint32_t)(uintptr_t)(dst0 + (wave + 4 * u) * 1024);
-                asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
-                             : "=&s"(m0_saved)
-                             : "s"(dst), "v"(off), "s"(tb)
-                             : "memory");
+                tiles::load_to_lds((uint32_t)(uintptr_t)(dst0 + (wave + 4 * u) * 1024), tb, off);
             }
         }
     };
     // wait until none of this wave's vector-memory operations is outstanding
-    auto wait_all = [&]() __attribute__((always_inline)) { __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); };
+    auto wait_all = [&]() __attribute__((always_inline)) { tiles::wait_vm<0>(); };
 
     // per-lane LDS read offsets
     // K (A operand): row = key (mbk * 32 + l32), chunk = t * 2 + half

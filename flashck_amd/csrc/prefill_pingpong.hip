@@ -23,6 +23,7 @@
 //   the second.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "lds_tiles.hpp"
 
 #include <type_traits>
 
@@ -43,25 +44,8 @@ struct PPShape {
     static_assert(TILEB % 8192 == 0, "a tile is split evenly over the 8 waves");
 };
 
-// XOR swizzles of the 16-byte chunk index.  They keep both LDS read patterns free of bank conflicts whether the LDS
-// serves 128 or 256 bytes per clock: K is read by 8/16 consecutive lanes = consecutive rows at one logical chunk; V by
-// 16/32 lanes = 4 rows x (2 or 4) adjacent chunks.
-template <int D>
-__device__ __forceinline__ int k_swz(int row)
-{
-    if constexpr (D >= 128)
-        return row & 15;
-    else
-        return ((row & 7) + ((row >> 3) & 1)) & 7;
-}
-template <int D>
-__device__ __forceinline__ int v_swz(int row, int lc)
-{
-    if constexpr (D >= 128)
-        return ((row & 3) << 1) ^ (((lc >> 1) & 1) << 3);
-    else
-        return (row & 3) << 1;
-}
+using tiles::k_swz;
+using tiles::v_swz;
 
 template <typename T, int D, int BN, bool kUniformPage>
 __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
@@ -173,46 +157,13 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         const int pc = (off % S::ROWB) >> 4;
         cp_row[u] = row;
         cp_k[u] = (pc ^ k_swz<D>(row)) * 8;
-        const int t = pc ^ ((row & 3) << 1);
-        cp_v[u] = (D >= 128 ? (t ^ (((t >> 1) & 1) << 3)) : t) * 8;  // inverse of lc -> lc ^ v_swz(row, lc)
+        cp_v[u] = tiles::v_chunk_at<D>(row, pc) * 8;
     }
 
-    // First cache row of every tile (uniform-page path): computed once per workgroup into LDS, so the main loop needs
-    // one LDS read per tile and no table lookup; tiles past the first kPrefillPageCache of a very long sequence are
-    // looked up one by one (tile_row0).
-    constexpr int kPageCache = kPrefillPageCache;
-    int FCK_LDS* row_lds = (int FCK_LDS*)(lds + 2 * kRing * S::TILEB);
-    if constexpr (kUniformPage) {
-        if (ks.table != nullptr)
-            for (int i = tid; i < min(n, kPageCache); i += 512) {
-                const int kb = (t_begin + i) * S::BN;
-                const int pi = a.kv.page_shift >= 0 ? kb >> a.kv.page_shift : kb / a.kv.page_size;
-                row_lds[i] = ks.table[pi] * a.kv.page_size + (kb - pi * a.kv.page_size);
-            }
-    }
-    // Lane l keeps the first row of tile row_chunk * 64 + l in a register; a lookup is then a v_readlane, and LDS is
-    // read once per 64 tiles (an LDS read in every phase would queue behind the operand reads of the matrix phase).
-    int row_vec = 0, row_chunk = -1;
-    auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t {
-        if (ks.table != nullptr) {
-            if (i >= kPageCache) {
-                // A sequence with more key tiles than the cache holds (> kPageCache * 64 keys): one table lookup per
-                // tile for the tiles past the cached ones.  A scalar load through the constant address space (the table
-                // is an input, never written here), consumed inside this branch so that the wait it needs stays here.
-                const int kb = (t_begin + i) * S::BN;
-                const int pi = a.kv.page_shift >= 0 ? kb >> a.kv.page_shift : kb / a.kv.page_size;
-                int page = ((const __attribute__((address_space(4))) int32_t*)ks.table)[pi];
-                asm volatile("" : "+s"(page));
-                return (int64_t)page * a.kv.page_size + (kb - pi * a.kv.page_size);
-            }
-            if ((i >> 6) != row_chunk) {
-                row_chunk = i >> 6;
-                row_vec = row_lds[min(row_chunk * 64 + lane, kPageCache - 1)];
-            }
-            return __builtin_amdgcn_readlane(row_vec, i & 63);
-        }
-        return ks.base_row + (t_begin + i) * S::BN;
-    };
+    // First cache row of every tile (uniform-page path), cached per workgroup (see tiles::FirstRows)
+    tiles::FirstRows<S::BN> first_rows{(int FCK_LDS*)(lds + 2 * kRing * S::TILEB)};
+    if constexpr (kUniformPage) first_rows.fill(a.kv, ks, t_begin, n, tid, 512);
+    auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t { return first_rows.row0(a.kv, ks, t_begin, i, lane); };
     auto tile = [&](int i) __attribute__((always_inline)) { return min(i, n - 1); };  // requests past the end re-read the last tile
     // request this wave's share of local tile `want` into ring buffer want % kRing (past the last tile: that tile
     // again); row0 = tile_row0(tile(want)) on the uniform-page path
@@ -224,32 +175,17 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
 #pragma unroll
         for (int u = 0; u < S::LD; ++u) {
             const int row = min(cp_row[u], room);  // rows past the last key repeat it (their scores are masked)
-            // Written as assembly on purpose: a load the compiler knows about makes it drain the whole load queue
-            // before the next LDS read it cannot prove disjoint.  m0 carries the LDS address of the block and is
-            // put back afterwards, since the compiler does not expect it to change.
-            uint32_t m0_saved;
             const uint32_t dst = (uint32_t)(uintptr_t)(ring + slot_ * S::TILEB + (wave + 8 * u) * 1024);
             if constexpr (kUniformPage) {
                 const uint16_t* tb = base + (row0 * row_stride + hkv * D);
-                const uint32_t off = (uint32_t)(row * (int)row_stride + cp_c[u]) * 2u;
-                asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
-                             : "=&s"(m0_saved)
-                             : "s"(dst), "v"(off), "s"(tb)
-                             : "memory");
+                tiles::load_to_lds(dst, tb, (uint32_t)(row * (int)row_stride + cp_c[u]) * 2u);
             } else {
-                const uint16_t* src = base + kv_row(a.kv, ks, kb + row) * row_stride + hkv * D + cp_c[u];
-                asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
-                             : "=&s"(m0_saved)
-                             : "s"(dst), "v"(src)
-                             : "memory");
+                tiles::load_to_lds(dst, base + kv_row(a.kv, ks, kb + row) * row_stride + hkv * D + cp_c[u]);
             }
         }
     };
     // wait until at most `keep` of this wave's vector-memory operations are outstanding (they complete in order)
-    auto wait_vm = [&](auto keep) __attribute__((always_inline)) {
-        constexpr int N = decltype(keep)::value;
-        __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-    };
+    auto wait_vm = [&](auto keep) __attribute__((always_inline)) { tiles::wait_vm<decltype(keep)::value>(); };
 
     // per-lane LDS read offsets
     // K (A operand): row = key (mbk * 32 + l32), chunk = t * 2 + half
