@@ -127,6 +127,9 @@ int main(int argc, char** argv)
     attn_case<bf16>("attn_bf16_causal_sq_gt_sk", 2, 11, 6, 32, 32, 1.f / std::sqrt(32.f), 2, -1, 0, g);
     attn_case<fp16>("attn_fp16_nomask", 4, 16, 16, 64, 64, 0.125f, 0, -1, -1, g);
     attn_case<fp16>("attn_fp16_window_tl", 2, 10, 17, 32, 32, 1.f / std::sqrt(32.f), 1, 4, 2, g);
+    // qk_head_dim != v_head_dim, head dims off the 64 / 128 / 256 grid (appended last: the records above keep their bytes)
+    attn_case<bf16>("attn_bf16_d40_dv72_causal_br", 2, 9, 14, 40, 72, 1.f / std::sqrt(40.f), 2, -1, 0, g);
+    attn_case<fp16>("attn_fp16_d192_dv128_nomask", 2, 5, 11, 192, 128, 1.f / std::sqrt(192.f), 0, -1, -1, g);
     fclose(g_out);
     return 0;
 }

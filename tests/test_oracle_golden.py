@@ -19,7 +19,7 @@ def test_rope_bit_exact(orc, tag, mode):
 
 
 ATTN = ["attn_bf16_nomask", "attn_bf16_causal_br", "attn_bf16_causal_tl", "attn_bf16_window_br", "attn_bf16_causal_sq_gt_sk",
-        "attn_fp16_nomask", "attn_fp16_window_tl"]
+        "attn_fp16_nomask", "attn_fp16_window_tl", "attn_bf16_d40_dv72_causal_br", "attn_fp16_d192_dv128_nomask"]
 
 
 @pytest.mark.parametrize("tag", ATTN)
