@@ -1,5 +1,6 @@
-"""Host model of every global -> LDS request the ping-pong prefill kernel issues (prefill_pingpong.hip): 64-bit tile
-base + 32-bit per-lane byte offset, the row clamp on the last tile of a sequence and the re-requests past the last tile.
+"""Host model of every global -> LDS request the two direct-to-LDS prefill kernels issue (prefill_pingpong.hip at head
+dims 64 / 128, prefill_dma.hip at head dim 256): 64-bit tile base + 32-bit per-lane byte offset, the row clamp on the
+last tile of a sequence and the re-requests past the last tile.
 
 For every workload the GPU tests run through these kernels (and for config 5 at full size) it asserts, for every
 workgroup, wave, instruction and lane:
@@ -202,3 +203,119 @@ def test_the_model_rejects_wrong_address_arithmetic():
     pool.page = pool.page * 2                    # first row = page id * wrong page size
     with pytest.raises(AssertionError):
         run_pingpong(pool, lanes)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# prefill_dma.hip (head dim 256): 4 waves, 128-row workgroups, two buffers per operand; wave w fills the 1 KiB blocks
+# w, w+4, ... of a tile (two rows each), so three offset registers serve all 16 instructions of a tile and the 8u rows
+# of block u go into the scalar base when every row of the tile exists.
+# ---------------------------------------------------------------------------------------------------------------------
+DMA_BM, DMA_D, DMA_LD = 128, 256, 64 * 512 // 1024 // 4
+
+
+def dma_lanes():
+    """(cp_row0, cp_pc, cp_kc0, cp_kc1, cp_vc) for every (wave, lane) of the 4-wave kernel"""
+    wave, lane = np.meshgrid(np.arange(4), np.arange(64), indexing="ij")
+    cp_row0 = wave * 2 + (lane >> 5)
+    cp_pc = lane & 31
+    cp_kc0 = (cp_pc ^ (cp_row0 & 15)) * 8
+    cp_kc1 = (cp_pc ^ ((cp_row0 + 8) & 15)) * 8
+    t = cp_pc ^ ((cp_row0 & 3) << 1)
+    cp_vc = (t ^ (((t >> 1) & 1) << 3)) * 8
+    return wave.ravel(), lane.ravel(), cp_row0.ravel(), cp_kc0.ravel(), cp_kc1.ravel(), cp_vc.ravel()
+
+
+def test_dma_kernel_swizzle_is_the_inverse_of_the_read_side():
+    """The three offset registers are enough: block w + 4u holds rows cp_row0 + 8u, whose K swizzle alternates with the
+    parity of u and whose V swizzle does not depend on u; every (row, chunk) lands once where its reader looks."""
+    D, CH = DMA_D, DMA_D // 8
+    wave, lane, cp_row0, kc0, kc1, vc = dma_lanes()
+    k_placed, v_placed, offs = {}, {}, []
+    for u in range(DMA_LD):
+        lds_off = (wave + 4 * u) * 1024 + lane * 16
+        row = cp_row0 + 8 * u
+        assert (lds_off // 512 == row).all() and ((lds_off % 512) >> 4 == (lane & 31)).all()
+        kc = kc1 if u & 1 else kc0
+        for r, ck, cv, o in zip(row, kc, vc, lds_off):
+            k_placed[(int(r), int(ck) // 8)] = int(o)
+            v_placed[(int(r), int(cv) // 8)] = int(o)
+        offs += lds_off.tolist()
+    assert sorted(offs) == list(range(0, BN * D * 2, 16)), "the 4 waves fill the tile exactly once"
+    assert len(k_placed) == BN * CH and len(v_placed) == BN * CH
+    for r in range(BN):
+        for lc in range(CH):
+            assert k_placed[(r, lc)] == r * 512 + ((lc ^ k_swz(D, r)) << 4)
+            assert v_placed[(r, lc)] == r * 512 + ((lc ^ v_swz(D, r, lc)) << 4)
+
+
+def dma_workgroups(pool):
+    """(b, hkv, t_begin, n) of every workgroup of the DMA kernel's 1-D grid (128-row tiles aligned to the sequence end)"""
+    g = pool.hq // pool.hk
+    groups = len(pool.lens) * pool.hk
+    gx = (groups + XCD - 1) // XCD
+    m_tiles = (max(pool.lens) + DMA_BM - 1) // DMA_BM
+    for bid in range(XCD * m_tiles * gx * g):
+        xcd, slot = bid % XCD, bid // XCD
+        gk, mt = (slot // g) % gx, m_tiles - 1 - slot // (g * gx)
+        gid = gk * XCD + xcd
+        if gid >= groups:
+            continue
+        b, hkv = gid // pool.hk, gid % pool.hk
+        sq = pool.lens[b]
+        tiles_b = (sq + DMA_BM - 1) // DMA_BM
+        if mt >= tiles_b:
+            continue
+        m0 = mt * DMA_BM - (tiles_b * DMA_BM - sq)
+        last_row = min(m0 + DMA_BM, sq) - 1
+        yield b, hkv, 0, max(0, (min(sq, last_row + 1) + BN - 1) // BN)
+
+
+def run_dma(pool):
+    wave, lane, cp_row0, kc0, kc1, vc = dma_lanes()
+    total = 0
+    for b, hkv, t_begin, n in dma_workgroups(pool):
+        if n <= 0:
+            continue
+        sk = pool.lens[b]
+        tiles = np.arange(n)                                    # request(0), then request(i + 1) while i + 1 < n
+        row0 = pool.first_rows(b, t_begin, n)
+        room = sk - 1 - (t_begin + tiles) * BN
+        assert room.min() >= 0
+        tile_off = row0 * pool.row_stride + hkv * pool.D        # elements
+        for u in range(DMA_LD):
+            for chunk in ((kc1 if u & 1 else kc0), vc):
+                # whole tiles: rows 8u.. go into the scalar base, the lane offset is cp_row0 * row_stride + chunk
+                off_whole = (cp_row0 * pool.row_stride + chunk) * 2
+                assert off_whole.max() < 2 ** 32
+                whole = room >= BN - 1
+                if whole.any():
+                    tb = (tile_off[whole] + 8 * u * pool.row_stride) * 2
+                    assert tb.min() + off_whole.min() >= 0 and tb.max() + off_whole.max() + 16 <= pool.pool_bytes
+                for t_off, rm in zip(tile_off[~whole], room[~whole]):
+                    off = (np.minimum(cp_row0 + 8 * u, rm) * pool.row_stride + chunk) * 2
+                    assert off.max() < 2 ** 32 and t_off * 2 + off.min() >= 0 and t_off * 2 + off.max() + 16 <= pool.pool_bytes
+        total += n
+    return total
+
+
+DMA_WORKLOADS = {
+    "midsize_every_row_d256": dict(lens=[5000, 300], hq=2, hk=1, head_dim=256),
+    "small_page64_d256": dict(seed=50 + 256 + 64, batch=5, hq=4, hk=2, head_dim=256, min_len=1, max_len=400, page_size=64),
+    "ragged_d256": dict(lens=[1, 63, 64, 65, 127, 128, 129, 255, 257, 513, 1024, 1500], hq=4, hk=2, head_dim=256),
+    "config5_d256": dict(head_dim=256),
+}
+
+
+@pytest.mark.parametrize("name", list(DMA_WORKLOADS))
+def test_every_request_of_the_dma_kernel_stays_inside_the_pool(name):
+    kw = dict(DMA_WORKLOADS[name])
+    pool = Pool(layout_only(**kw), 256)
+    assert run_dma(pool) > 0
+
+
+def test_the_dma_model_rejects_wrong_address_arithmetic():
+    pool = Pool(layout_only(lens=[700, 300], hq=8, hk=2, head_dim=256), 256)
+    assert run_dma(pool) > 0
+    pool.row_stride = pool.hq * pool.D          # the mistake: query heads instead of KV heads
+    with pytest.raises(AssertionError):
+        run_dma(pool)
