@@ -1,7 +1,7 @@
 """Shared helpers of the parity tests."""
 import torch
 
-# BASELINE tolerances: max-abs error of attention outputs against the fp32-accumulated reference
+# Tolerances of the parity tests: max-abs error of attention outputs against the fp32-accumulated reference
 ATOL = {torch.float16: 1e-2, torch.bfloat16: 2e-2}
 
 
