@@ -68,12 +68,12 @@ __device__ __forceinline__ void wait_vm()
 }
 
 // First cache row of key tile i (BN keys, local index from t_begin) of a paged sequence whose tiles never straddle a
-// page.  fill() computes the first kPrefillPageCache of them once per workgroup into LDS (a barrier must follow); row0()
+// page.  fill() computes the first CACHE of them once per workgroup into LDS (a barrier must follow); row0()
 // then costs a v_readlane: lane l keeps the entry of tile chunk * 64 + l in a register and LDS is read once per 64
 // tiles (an LDS read per tile would queue behind the operand reads of the matrix work).  Tiles past the cached ones of
 // a very long sequence are looked up one by one, with a scalar load through the constant address space (the table is
 // an input, never written here) that is consumed on the spot, so that the wait it needs stays there.
-template <int BN>
+template <int BN, int CACHE = kPrefillPageCache>
 struct FirstRows {
     int FCK_LDS* rows;
     int vec = 0, chunk = -1;
@@ -86,12 +86,12 @@ struct FirstRows {
     __device__ __forceinline__ void fill(const KvAddr& kv, const KvSeq& ks, int t_begin, int n, int tid, int nthreads)
     {
         if (ks.table != nullptr)
-            for (int i = tid; i < min(n, kPrefillPageCache); i += nthreads) rows[i] = table_row(kv, ks.table, (t_begin + i) * BN);
+            for (int i = tid; i < min(n, CACHE); i += nthreads) rows[i] = table_row(kv, ks.table, (t_begin + i) * BN);
     }
     __device__ __forceinline__ int64_t row0(const KvAddr& kv, const KvSeq& ks, int t_begin, int i, int lane)
     {
         if (ks.table != nullptr) {
-            if (i >= kPrefillPageCache) {
+            if (i >= CACHE) {
                 const int kb = (t_begin + i) * BN;
                 const int pi = kv.page_shift >= 0 ? kb >> kv.page_shift : kb / kv.page_size;
                 int page = ((const __attribute__((address_space(4))) int32_t*)ks.table)[pi];
@@ -100,7 +100,7 @@ struct FirstRows {
             }
             if ((i >> 6) != chunk) {
                 chunk = i >> 6;
-                vec = rows[min(chunk * 64 + lane, kPrefillPageCache - 1)];
+                vec = rows[min(chunk * 64 + lane, CACHE - 1)];
             }
             return __builtin_amdgcn_readlane(vec, i & 63);
         }
