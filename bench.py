@@ -350,7 +350,8 @@ def main():
     line = {
         "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic", "config": {"workload": name, "kv_pool_copies_rotated": args.copies},
+        "data": "synthetic", "config": {"workload": name, "kv_pool_copies_rotated": args.copies,
+                                "library": os.path.relpath(_lib.LIB_PATH, ROOT)},
         "roofline": roof, "cpu_baseline": cpu, "extra": extra,
     }
     print(json.dumps(line))

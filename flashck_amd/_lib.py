@@ -7,8 +7,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# FLASHCK_FMHA_LIB points at another build of the same library (for example one compiled with different tuning macros)
-LIB_PATH = os.environ.get("FLASHCK_FMHA_LIB") or os.path.join(_HERE, "libflashck_fmha.so")
+# the one library the operators use: the in-tree build next to this file (no environment override)
+LIB_PATH = os.path.join(_HERE, "libflashck_fmha.so")
 
 _vp, _i64, _i32, _u32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_uint32, ctypes.c_float
 

@@ -59,7 +59,10 @@ def build(verbose=False, extra_flags=()):
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}")
     os.replace(tmp, LIB)
-    build_header_test()
+    try:
+        build_header_test()
+    except RuntimeError as e:  # a test program that does not build must not take the library down with it
+        print(f"warning: {e}", file=sys.stderr)
     return LIB
 
 

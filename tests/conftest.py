@@ -27,4 +27,7 @@ def fmha():
     from flashck_amd.ops import fmha as ops
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     _lib.load()
+    # the library under test is the in-tree build, never another copy
+    want = os.path.join(ROOT, "flashck_amd", "libflashck_fmha.so")
+    assert os.path.realpath(_lib.LIB_PATH) == os.path.realpath(want), f"tests loaded {_lib.LIB_PATH}, not {want}"
     return ops
