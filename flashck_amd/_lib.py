@@ -34,6 +34,8 @@ SIGNATURES = {
     "fck_fmha_fwd_pagedkv_attrs": (ctypes.c_int, [_vp] * 7 + [_i64] * 9 + [_f32, _i64, _i64, _u32, _i32, _ap, _vp]),
     "fck_fmha_fwd_splitkv": (ctypes.c_int, [_vp] * 11 + [_i64] * 11 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_fwd_splitkv_fused": (ctypes.c_int, [_vp] * 10 + [_i64] * 11 + [_f32, _i64, _i64, _u32, _i32, _vp]),
+    "fck_fmha_fused_reset": (ctypes.c_int, [_vp]),
+    "fck_fmha_validate_paged": (ctypes.c_int, [_vp] * 6 + [_i64] * 3 + [_vp, _vp]),
     "fck_fmha_fwd_splitkv_combine": (ctypes.c_int, [_vp] * 4 + [_i64] * 6 + [_i32, _vp]),
     "fck_fmha_fwd_appendkv": (ctypes.c_int, [_vp] * 7 + [_i64, _vp, _vp, _i64, _i32, _i32, _vp, _i64, _i64, _vp]
                               + [_i64] * 6 + [_i32, _vp]),

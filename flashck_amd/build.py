@@ -16,7 +16,7 @@ OBJ = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libflashck_fmha.so")
 
 SOURCES = ["fmha_api.cpp", "splitkv_decode.hip", "splitkv_combine.hip", "appendkv_rope.hip", "prefill.hip",
-           "prefill_pingpong.hip", "prefill_dma.hip"]
+           "prefill_pingpong.hip", "prefill_dma.hip", "validate.hip"]
 
 FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "--offload-arch=gfx950", "-fno-gpu-rdc",

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "gfx950_ops.hpp"
+
 namespace fck {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -17,8 +19,6 @@ typedef short s16x8_t __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
-
-#define FCK_LDS __attribute__((address_space(3)))
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -103,23 +103,7 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(const void FCK_LDS* p)
     return __builtin_bit_cast(u32x2_t, v);
 }
 
-// Cross-lane reductions on the VALU (v_permlane16_swap / v_permlane32_swap, no LDS round trip).
-// v_permlane32_swap a, b exchanges lanes 32..63 of a with lanes 0..31 of b; v_permlane16_swap does the same between the
-// odd 16-lane rows of a and the even rows of b.  Started from two copies of x they leave (x[l % 32], x[l % 32 + 32]) resp.
-// (x[even row of l], x[odd row of l]) in every lane.  The instructions are written as inline assembly because they
-// update both operands in place; the s_nop covers the wait states a VALU write needs before a lane permute reads it.
-__device__ __forceinline__ void swap32(float x, float& a, float& b)
-{
-    a = x;
-    b = x;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-}
-__device__ __forceinline__ void swap16(float x, float& a, float& b)
-{
-    a = x;
-    b = x;
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-}
+// Cross-lane reductions on the VALU (swap32 / swap16 of gfx950_ops.hpp).
 // over the lane pair (l, l ^ 32)
 __device__ __forceinline__ float pair32_max(float x)
 {

@@ -122,17 +122,19 @@ int launch_status(hipError_t e, const char* what)
     return FCK_OK;
 }
 
+// compute units of the current device (looked up once per device)
 int cu_count()
 {
-    static int cus = 0;
-    static std::once_flag once;
-    std::call_once(once, [] {
-        int dev = 0;
+    constexpr int kMaxDev = 64;
+    static int cus[kMaxDev];
+    static std::once_flag once[kMaxDev];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 256;
+    std::call_once(once[dev], [dev] {
         hipDeviceProp_t p;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
-        if (cus <= 0) cus = 256;
+        cus[dev] = hipGetDeviceProperties(&p, dev) == hipSuccess && p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
     });
-    return cus;
+    return cus[dev];
 }
 
 }  // namespace
@@ -352,6 +354,42 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
     g_kernel = uniform ? "splitkv_decode_kernel<uniform_page,fused>" : "splitkv_decode_kernel<row_lookup,fused>";
     return launch_status(fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
                          "FmhaFwdSplitKV (fused) launch");
+}
+
+int fck_fmha_fused_reset(void* stream)
+{
+    g_err[0] = 0;
+    float* scratch = nullptr;
+    if (hipError_t e = fck::decode_scratch(&scratch); e != hipSuccess) return launch_status(e, "scratch symbol lookup");
+    return launch_status(fck::launch_clear_tickets(reinterpret_cast<uint32_t*>(scratch), (int)fck::kDecodeScratchTickets, static_cast<hipStream_t>(stream)),
+                         "ticket reset launch");
+}
+
+int fck_fmha_validate_paged(const int32_t* seqlen_k, const int32_t* block_table, int64_t batch_stride_block_table,
+                            const int32_t* kv_indptr, const int32_t* kv_page_indices, const int32_t* kv_last_page_lens,
+                            int64_t batch, int64_t num_total_pages, int64_t page_block_size, int32_t* error_counts, void* stream)
+{
+    g_err[0] = 0;
+    if (batch <= 0 || num_total_pages <= 0 || page_block_size <= 0 || batch > INT32_MAX || page_block_size > INT32_MAX)
+        return fail(FCK_ERR_INVALID_ARGUMENT, "batch, num_total_pages and page_block_size must be positive");
+    if (!error_counts) return fail(FCK_ERR_INVALID_ARGUMENT, "error_counts (int32[4], device memory) must not be null");
+    if ((block_table != nullptr) == (kv_indptr != nullptr))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "give either a block table (with seqlen_k) or a page list (kv_indptr, kv_page_indices)");
+    if (block_table && (!seqlen_k || batch_stride_block_table <= 0))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "a block table needs seqlen_k and batch_stride_block_table > 0");
+    if (kv_indptr && !kv_page_indices) return fail(FCK_ERR_INVALID_ARGUMENT, "a page list needs kv_page_indices");
+    fck::ValidateArgs a{};
+    a.seqlen_k = seqlen_k;
+    a.block_table = block_table;
+    a.block_table_stride = batch_stride_block_table;
+    a.kv_indptr = kv_indptr;
+    a.kv_page_indices = kv_page_indices;
+    a.kv_last_page_lens = kv_last_page_lens;
+    a.num_total_pages = num_total_pages;
+    a.page_size = (int32_t)page_block_size;
+    a.batch = (int32_t)batch;
+    a.counts = error_counts;
+    return launch_status(fck::launch_validate_paged(a, static_cast<hipStream_t>(stream)), "paged-cache validation launch");
 }
 
 int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o, const int32_t* seqstart_q, int64_t batch,

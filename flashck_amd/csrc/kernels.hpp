@@ -96,6 +96,22 @@ struct PrefillArgs {
     int32_t d, dv;  // head dims of Q/K and of V/O as stored; other than the kernel's D only in the 4-wave kernel of prefill.hip
 };
 
+// arguments of the paged-cache checker: a block table (block_table != nullptr: seqlen_k, block_table_stride) or a page
+// list (kv_indptr, kv_page_indices, optional kv_last_page_lens)
+struct ValidateArgs {
+    const int32_t* seqlen_k;
+    const int32_t* block_table;
+    int64_t block_table_stride;
+    const int32_t* kv_indptr;
+    const int32_t* kv_page_indices;
+    const int32_t* kv_last_page_lens;
+    int64_t num_total_pages;
+    int32_t page_size, batch;
+    int32_t* counts;  // int32[4], device memory of the caller
+};
+hipError_t launch_validate_paged(const ValidateArgs& a, hipStream_t st);
+hipError_t launch_clear_tickets(uint32_t* tickets, int n, hipStream_t st);
+
 hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page, int num_cu,
                                  hipStream_t st);
 // Device memory the fused split-KV entry point uses instead of a caller-owned workspace: a fixed array in the library

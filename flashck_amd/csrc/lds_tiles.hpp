@@ -1,6 +1,6 @@
 // Tile machinery shared by the prefill kernels that send K/V tiles global -> LDS directly (prefill_pingpong.hip,
-// prefill_dma.hip): the XOR swizzles of a staged tile, the global -> LDS instruction, the wait on a wave's own loads and
-// the per-workgroup cache of every key tile's first cache row.
+// prefill_dma.hip): the XOR swizzles of a staged tile and the per-workgroup cache of every key tile's first cache
+// row (the global -> LDS instruction itself and the wait on a wave's own loads are in gfx950_ops.hpp).
 #pragma once
 #include "common.hpp"
 #include "kernels.hpp"
@@ -37,35 +37,8 @@ __device__ __forceinline__ int v_chunk_at(int row, int pc)
     return D >= 128 ? (t ^ (((t >> 1) & 1) << 3)) : t;
 }
 
-// One global -> LDS instruction: every lane copies 16 bytes from base + off (base uniform, off per lane, in bytes) to
-// the 1 KiB block at LDS address dst (uniform), lane l to byte l*16 of it.  Written as assembly on purpose: a load the
-// compiler knows about makes it drain the whole load queue before the next LDS read it cannot prove disjoint, and no
-// register is a load destination, so nothing the compiler schedules can wait on these loads by accident.  m0 carries
-// the LDS address and is put back afterwards, since the compiler does not expect it to change.
-__device__ __forceinline__ void load_to_lds(uint32_t dst, const void* base, uint32_t off)
-{
-    uint32_t m0_saved;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
-                 : "=&s"(m0_saved)
-                 : "s"(dst), "v"(off), "s"(base)
-                 : "memory");
-}
-// the same with a full address per lane
-__device__ __forceinline__ void load_to_lds(uint32_t dst, const void* src)
-{
-    uint32_t m0_saved;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
-                 : "=&s"(m0_saved)
-                 : "s"(dst), "v"(src)
-                 : "memory");
-}
-
-// wait until at most N of this wave's vector-memory operations are outstanding (they complete in order)
-template <int N>
-__device__ __forceinline__ void wait_vm()
-{
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
+using fck::load_to_lds;
+using fck::wait_vm;
 
 // First cache row of key tile i (BN keys, local index from t_begin) of a paged sequence whose tiles never straddle a
 // page.  fill() computes the first CACHE of them once per workgroup into LDS (a barrier must follow); row0()
@@ -94,8 +67,8 @@ struct FirstRows {
             if (i >= CACHE) {
                 const int kb = (t_begin + i) * BN;
                 const int pi = kv.page_shift >= 0 ? kb >> kv.page_shift : kb / kv.page_size;
-                int page = ((const __attribute__((address_space(4))) int32_t*)ks.table)[pi];
-                asm volatile("" : "+s"(page));
+                int page = const_load(ks.table, pi);
+                FCK_PIN_SGPR(page);
                 return (int64_t)page * kv.page_size + (kb - pi * kv.page_size);
             }
             if ((i >> 6) != chunk) {

@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
     const int dvs = kPad ? a.dv : D;  // elements per stored V / O row
     typedef PrefillShape<D> S;
     typedef typename T::vec8 vec8;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    FCK_DYNAMIC_LDS(smem);
     char FCK_LDS* lds = (char FCK_LDS*)smem;  // K0 | K1 | V0 | V1
 
     const int tid = threadIdx.x;

@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     typedef Shape<D> S;
     typedef typename T::vec8 vec8;
     constexpr int BN = S::BN;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    FCK_DYNAMIC_LDS(smem);
     char FCK_LDS* lds = (char FCK_LDS*)smem;  // K0 | K1 | V0 | V1 | first rows (kPrefillPageCache x int32)
     int FCK_LDS* const row_lds = (int FCK_LDS*)(lds + 4 * S::TILEB);
 
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
                     const int row = min(cp_row0 + 8 * u, room);
                     off = (uint32_t)(row * (int)row_stride + (kv == 0 ? ((u & 1) ? cp_kc1 : cp_kc0) : cp_vc)) * 2u;
                 }
-                tiles::load_to_lds((uint32_t)(uintptr_t)(dst0 + (wave + 4 * u) * 1024), tb, off);
+                tiles::load_to_lds(lds_address(dst0 + (wave + 4 * u) * 1024), tb, off);
             }
         }
     };
@@ -245,12 +245,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
 #pragma unroll
             for (int q = 0; q < S::DVB; ++q)
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    float x;
-                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(oacc[q][j]));
-                    x *= alpha;
-                    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(oacc[q][j]) : "v"(x));
-                }
+                for (int j = 0; j < 16; ++j) FCK_ACC_SCALE(oacc[q][j], alpha);
         }
         const float m_ref = (m_run == -INFINITY) ? 0.f : m_run;
         float psum = 0.f;

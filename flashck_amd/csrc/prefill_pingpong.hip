@@ -54,7 +54,7 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     typedef typename T::vec8 vec8;
     static_assert(S::NB == 2, "the matrix phase is written for 64-key tiles");
     constexpr int kRing = S::RING;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    FCK_DYNAMIC_LDS(smem);
     char FCK_LDS* lds = (char FCK_LDS*)smem;  // K ring | V ring | page ids (kPrefillPageCache x int32)
     char FCK_LDS* const k_ring = lds;
     char FCK_LDS* const v_ring = lds + kRing * S::TILEB;
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
 #pragma unroll
         for (int u = 0; u < S::LD; ++u) {
             const int row = min(cp_row[u], room);  // rows past the last key repeat it (their scores are masked)
-            const uint32_t dst = (uint32_t)(uintptr_t)(ring + slot_ * S::TILEB + (wave + 8 * u) * 1024);
+            const uint32_t dst = lds_address(ring + slot_ * S::TILEB + (wave + 8 * u) * 1024);
             if constexpr (kUniformPage) {
                 const uint16_t* tb = base + (row0 * row_stride + hkv * D);
                 tiles::load_to_lds(dst, tb, (uint32_t)(row * (int)row_stride + cp_c[u]) * 2u);
@@ -319,8 +319,8 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         // are sunk past it into the matrix phase and the two wave groups stop overlapping.
 #pragma unroll
         for (int ks4 = 0; ks4 < 2 * S::NB; ++ks4)
-            asm volatile("" : "+v"(pfrag[ks4][0]), "+v"(pfrag[ks4][1]), "+v"(pfrag[ks4][2]), "+v"(pfrag[ks4][3]));
-        asm volatile("" : "+v"(l_run));
+            FCK_PIN_VGPR4(pfrag[ks4][0], pfrag[ks4][1], pfrag[ks4][2], pfrag[ks4][3]);
+        FCK_PIN_VGPR(l_run);
     };
 
     if (n > 0) {

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
     const int dvs = kPad ? a.dv : D;  // elements per stored V / partial-output row
     typedef DecodeShape<D, HG> S;
     typedef typename T::vec8 vec8;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    FCK_DYNAMIC_LDS(smem);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
                 const uint32_t e2 = __builtin_amdgcn_readlane(tbl_vec[2], pi >> 2), e3 = __builtin_amdgcn_readlane(tbl_vec[3], pi >> 2);
                 page = (int)((pi & 2) ? ((pi & 1) ? e3 : e2) : ((pi & 1) ? e1 : e0));
             } else {
-                page = ((const __attribute__((address_space(4))) int32_t*)ks.table)[pi];
+                page = const_load(ks.table, pi);
             }
             return (int64_t)page * a.kv.page_size + (kb - pi * a.kv.page_size);
         }
@@ -346,6 +346,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
 
     auto compute_tile = [&](int c) {
         const int kb = (t_begin + c) * S::TK;
+        FCK_WAVE_LDS_ORDER();  // the staging tile was written by all lanes of this wave; the reads below come after
 #pragma unroll
         for (int hl = 0; hl < HG; ++hl) {
             const char FCK_LDS* kh = kstage + hl * S::HTILE;

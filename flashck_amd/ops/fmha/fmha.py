@@ -18,14 +18,14 @@ from typing import Optional, Tuple
 import torch
 
 from ... import _lib
-from ...utils import FlashCKOperationType, register_flashck_functions, tuning
+from ...utils import FlashCKOperationType, flags, register_flashck_functions, tuning
 
 __all__ = [
     "MASK_NONE", "MASK_TOP_LEFT", "MASK_BOTTOM_RIGHT", "MASK_GENERIC", "ROPE_NONE", "ROPE_INTERLEAVED",
     "ROPE_HALF_ROTATED", "fmha_fwd", "fmha_fwd_varlen", "fmha_fwd_splitkv", "fmha_fwd_splitkv_combine",
     "fmha_fwd_splitkv_fused", "fused_splitkv_fits",
     "fmha_fwd_appendkv", "fmha_batch_prefill", "fmha_fwd_pagedkv", "fmha_decode_paged", "fmha_decode_step",
-    "tune_decode_num_splits", "DecodeWorkspace", "num_splits_heuristic", "splitkv_workspace",
+    "tune_decode_num_splits", "DecodeWorkspace", "num_splits_heuristic", "splitkv_workspace", "validate_paged", "fused_reset",
 ]
 
 # GenericAttentionMaskEnum / RopeEnum, core/profiling/attention/fmha_library.h:81-87,195-200
@@ -177,6 +177,51 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
     return ctypes.byref(a), (a, bias, alibi_slopes)
 
 
+def validate_paged(*, seqlen_k=None, block_table=None, kv_indptr=None, kv_page_indices=None, kv_last_page_lens=None,
+                   num_total_pages: int, page_size: int, out=None, check: bool = False):
+    """Debug aid: checks on the GPU what the paged kernels trust - key counts against what the block-table row / page
+    list can address, page ids against the pool - without allocating when `out` (int32[4] on the device) is given.
+    Returns the counters tensor [sequences with a bad length, page ids out of range, malformed page lists, first
+    offending sequence or -1]; nothing is read back unless check=True, which synchronises and raises ValueError when a
+    counter is non-zero.  The operators call it with check=True before every paged launch while the flag
+    FC_DEBUG_KERNEL_INSTANCE is on (core/utils/flags.cc:169)."""
+    paged = block_table is not None
+    ref = block_table if paged else kv_indptr
+    _check_tensor("block_table" if paged else "kv_indptr", ref, dtype=torch.int32, ndim=2 if paged else 1)
+    if paged:
+        _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1)
+        if kv_indptr is not None or kv_page_indices is not None:
+            raise ValueError("give a block table or a page list, not both")
+        B, stride = block_table.shape
+        if seqlen_k.numel() != B:
+            raise ValueError(f"seqlen_k has {seqlen_k.numel()} entries, the block table {B} rows")
+    else:
+        _check_tensor("kv_page_indices", kv_page_indices, dtype=torch.int32, ndim=1)
+        _check_tensor("kv_last_page_lens", kv_last_page_lens, dtype=torch.int32, ndim=1, optional=True)
+        B, stride = kv_indptr.numel() - 1, 0
+    counts = _out("out", out, (4,), torch.int32, ref)
+    _call("fck_fmha_validate_paged", _ptr(seqlen_k), _ptr(block_table), stride, _ptr(kv_indptr), _ptr(kv_page_indices),
+          _ptr(kv_last_page_lens), B, int(num_total_pages), int(page_size), _ptr(counts), _stream())
+    if check:
+        bad_len, bad_page, bad_list, first = counts.tolist()
+        if bad_len or bad_page or bad_list:
+            raise ValueError(f"paged-cache arguments are inconsistent: {bad_len} sequence(s) longer than their table can address, "
+                             f"{bad_page} page id(s) outside the pool of {num_total_pages}, {bad_list} malformed page list(s); "
+                             f"first offending sequence: {first}")
+    return counts
+
+
+def _debug_validate(**kw):
+    if flags.flag("FC_DEBUG_KERNEL_INSTANCE"):
+        validate_paged(check=True, **kw)
+
+
+def fused_reset() -> None:
+    """Zero the arrival tickets of fmha_fwd_splitkv_fused on the current device (after a fused launch that did not run
+    to completion; see fck_fmha_fused_reset)."""
+    _call("fck_fmha_fused_reset", _stream())
+
+
 def num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, num_cu=0) -> int:
     """Split count chosen from the CU count and the KV length."""
     return int(_lib.load().fck_fmha_num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k,
@@ -295,6 +340,7 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
         if block_table.dim() != 2 or block_table.shape[0] != B:
             raise ValueError(f"block_table must be [batch, max_pages_per_seq], got {tuple(block_table.shape)}")
         page, sk, max_blocks = k.shape[1], 0, block_table.numel()
+        _debug_validate(seqlen_k=seqlen_k, block_table=block_table, num_total_pages=k.shape[0], page_size=page)
     else:
         page, max_blocks = 0, 0
         sk = k.shape[0] if cu_seqlens_k is not None else k.shape[1]
@@ -375,6 +421,7 @@ def fmha_fwd_splitkv_fused(q, k, v, num_splits: int = 0, *, seqlen_k=None, block
         if block_table.dim() != 2 or block_table.shape[0] != B:
             raise ValueError(f"block_table must be [batch, max_pages_per_seq], got {tuple(block_table.shape)}")
         page, sk, max_blocks = k.shape[1], 0, block_table.numel()
+        _debug_validate(seqlen_k=seqlen_k, block_table=block_table, num_total_pages=k.shape[0], page_size=page)
     else:
         page, max_blocks = 0, 0
         sk = k.shape[0] if cu_seqlens_k is not None else k.shape[1]
@@ -462,6 +509,10 @@ def fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, *, cu_seqlens_k
         rotary_dim = 0
     if block_table is not None:
         stride, page, rows = block_table.shape[1], k_cache.shape[1], 0
+        if flags.flag("FC_DEBUG_KERNEL_INSTANCE"):  # the table must hold the sequences WITH their new tokens
+            grown = seqlen_k + ((cu_seqlens_knew[1:] - cu_seqlens_knew[:-1]) if packed else n)
+            validate_paged(seqlen_k=grown.to(torch.int32), block_table=block_table, num_total_pages=k_cache.shape[0],
+                           page_size=page, check=True)
     else:
         stride, page, rows = 0, 0, k_cache.shape[1]
     _call("fck_fmha_fwd_appendkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(knew), _ptr(vnew), _ptr(seqlen_k),
@@ -490,6 +541,8 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
     num_pages, page, Hk, Dv = v_cache.shape
     o = _out("out", out, (tq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
+    _debug_validate(kv_indptr=kv_indptr, kv_page_indices=kv_page_indices, kv_last_page_lens=kv_last_page_lens,
+                    num_total_pages=num_pages, page_size=page)
     at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1)
     if at is None:
         _call("fck_fmha_batch_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
@@ -527,6 +580,7 @@ def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q
         raise ValueError("group mode needs max_seqlen_q")
     o = _out("out", out, (*q.shape[:-1], Dv), q.dtype, q)
     wl, wr = _window(window)
+    _debug_validate(seqlen_k=seqlen_k, block_table=block_table, num_total_pages=k_cache.shape[0], page_size=page)
     at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, q.shape[0] if group else sq, 1)
     if at is None:
         _call("fck_fmha_fwd_pagedkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
@@ -547,6 +601,21 @@ def _auto_num_splits(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, h
         lambda: num_splits_heuristic(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim),
         batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size,
         "fp16" if dtype == torch.float16 else "bf16")
+
+
+def _usable_variant(variant, q_num_heads, kv_num_heads, rows, head_dim, v_head_dim, plain=True):
+    """A kernel variant from the tuning cache is a hint: the record's problem class is coarser than what the variant
+    needs (query counts are bucketed, v_head_dim is not part of the key), so its preconditions are checked again for
+    this call, and 0 (the library's choice) is returned when one fails.  Head pairs (2) need an even number of KV heads,
+    equal head dims of 64 or 128, at most 16 packed query rows (queries x heads per KV head) and no score modifier /
+    fp8 cache; one head per workgroup (1) fits every call."""
+    variant = int(variant)
+    if variant == 2:
+        g = q_num_heads // max(kv_num_heads, 1)
+        ok = (plain and kv_num_heads % 2 == 0 and head_dim == v_head_dim and head_dim in (64, 128)
+              and rows * g <= 16)
+        return 2 if ok else 0
+    return variant if variant == 1 else 0
 
 
 def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits: int = 0, max_seqlen_k: int = 0,
@@ -581,8 +650,8 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * k_cache.shape[1]
         num_splits, cached_variant = _auto_num_splits(B, Hq, Hk, sq, max_seqlen_k, D, k_cache.shape[1], q.dtype)
-        if not decode_variant and plain:
-            decode_variant = cached_variant
+        if not decode_variant:
+            decode_variant = _usable_variant(cached_variant, Hq, Hk, sq, D, v_cache.shape[3], plain)
     if fused:
         if not plain or decode_variant:
             raise NotImplementedError("the fused launch takes no bias / soft cap / fp8 cache / kernel variant")
@@ -703,6 +772,7 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * page  # what the block table can address
         num_splits, decode_variant = _auto_num_splits(B, Hq, Hk, n, max_seqlen_k, D, page, q.dtype)
+        decode_variant = _usable_variant(decode_variant, Hq, Hk, n, D, Dv)
     else:
         decode_variant = 0
     # a lone new token sees every key: no mask needed unless a sliding window is asked for

@@ -60,6 +60,8 @@ def _define(name, default, doc, writable=True):
 
 
 # names, defaults and help texts follow core/utils/flags.cc:157,201-233 unless noted
+# here: every paged launch of the Python operators is preceded by a device-side check of its block table / page list
+_define("FC_DEBUG_KERNEL_INSTANCE", False, "Enable kernel instance debugging")
 _define("FC_TUNING_DB_DIR", "", "Directory for profiler cache storage")
 _define("FC_FORCE_PROFILING", False, "Force profiling even if cached results exist")  # reference default: true
 _define("FC_FLUSH_PROFILING_DB", False, "Flush profile cache database on startup")

@@ -191,6 +191,34 @@ FCK_EXPORT int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const vo
                                           int32_t dtype, void* stream);
 
 /*
+ * Puts the arrival tickets of fck_fmha_fwd_splitkv_fused back to zero on the current device (one small fill launch on
+ * `stream`, nothing allocated).  The tickets reset themselves at the end of every fused launch that runs to
+ * completion; after a launch that did not (a device error, a cancelled graph launch) they may be left non-zero and
+ * every later fused call on that GPU would merge at the wrong moment: call this once before going on.  No counterpart
+ * in the reference.
+ */
+FCK_EXPORT int fck_fmha_fused_reset(void* stream);
+
+/*
+ * Debug aid: checks the paged-cache arguments that the attention kernels trust, on the GPU, without allocating and
+ * without reading anything back (the reference's debug aid for tensors is the validator of
+ * core/utils/debug_utils.cc:43-130; its FMHA glue has no such check).  Give either a block table
+ * (block_table int32 [B, batch_stride_block_table] with seqlen_k int32 [B]; the page-list pointers NULL) or a page
+ * list (kv_indptr int32 [B+1], kv_page_indices, optional kv_last_page_lens; block_table and seqlen_k NULL).
+ * error_counts: int32[4] in device memory of the caller, overwritten by one single-workgroup launch on `stream`:
+ *   [0] sequences whose key count is negative or larger than their table row / page list can address
+ *   [1] page ids outside [0, num_total_pages) among the table entries the sequences use
+ *   [2] malformed page lists (kv_indptr not monotone, kv_last_page_lens outside [1, page_block_size])
+ *   [3] index of the first offending sequence, -1 when there is none
+ * A kernel launched with arguments for which any of [0..2] is non-zero reads outside the cache.
+ */
+FCK_EXPORT int fck_fmha_validate_paged(const int32_t* seqlen_k, const int32_t* block_table,
+                                       int64_t batch_stride_block_table, const int32_t* kv_indptr,
+                                       const int32_t* kv_page_indices, const int32_t* kv_last_page_lens,
+                                       int64_t batch, int64_t num_total_pages, int64_t page_block_size,
+                                       int32_t* error_counts, void* stream);
+
+/*
  * LSE combine: O = sum_s exp(lse_acc[s] - logsumexp_s lse_acc) * o_acc[s], stored as T.
  * Replaces `FmhaSplitKVCombine` / `FmhaFwdSplitKVCombine`, fmha_fwd_split_kv_combine_jinja.h:78-92
  * (args :37-76, strides :114-165), declared at fmha_fwd_split_kv_combine_call.h:26-36.

@@ -12,6 +12,21 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_collection_modifyitems(config, items):
+    """tests/test_emu_kernels.py re-runs the GPU test functions on the CPU emulator; by default only the cases named in
+    tests/emu/quick_cases.txt (about two minutes in one process), all of them with FCK_EMU_FULL=1."""
+    if os.environ.get("FCK_EMU_FULL") == "1":
+        return
+    try:
+        with open(os.path.join(ROOT, "tests", "emu", "quick_cases.txt")) as f:
+            quick = {line.strip() for line in f if line.strip() and not line.startswith("#")}
+    except OSError:
+        quick = set()
+    for item in items:
+        if item.module.__name__ == "test_emu_kernels" and item.name not in quick:
+            item.add_marker(pytest.mark.skip(reason="not in the emulator's quick set; FCK_EMU_FULL=1 runs it"))
+
+
 @pytest.fixture(scope="session")
 def orc():
     from oracle import fmha_oracle

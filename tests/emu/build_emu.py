@@ -1,0 +1,49 @@
+"""Builds tests/emu/libflashck_fmha_emu.so: the kernel sources of flashck_amd/csrc, unchanged, compiled as C++ for the
+host on top of the wave64 emulator in this directory.  Test infrastructure: only tests load the result."""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+CSRC = os.path.join(ROOT, "flashck_amd", "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "libflashck_fmha_emu.so")
+CXX = "/opt/rocm/llvm/bin/clang++"
+
+sys.path.insert(0, ROOT)
+from flashck_amd.build import SOURCES  # noqa: E402  (the same translation units as the shipped library)
+
+FLAGS = ["-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off", "-mf16c", "-mavx2",
+         "-I", os.path.join(HERE, "include"), "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-I", HERE,
+         "-include", os.path.join(HERE, "include", "gfx950_ops.hpp"),
+         "-Wall", "-Wno-unused-function", "-Wno-unused-variable", "-Wno-unused-but-set-variable", "-Wno-unknown-pragmas"]
+
+
+def _compile(path):
+    obj = os.path.join(OBJ, os.path.splitext(os.path.basename(path))[0] + ".o")
+    if os.path.exists(obj) and os.path.getmtime(obj) > max(
+            os.path.getmtime(os.path.join(d, f)) for d in (CSRC, HERE, os.path.join(HERE, "include"), os.path.join(ROOT, "include", "flashck", "fmha"))
+            for f in os.listdir(d) if os.path.isfile(os.path.join(d, f))):
+        return obj
+    r = subprocess.run([CXX] + FLAGS + ["-c", path, "-o", obj], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"emulator build failed on {path}:\n{r.stdout[-6000:]}")
+    return obj
+
+
+def build():
+    os.makedirs(OBJ, exist_ok=True)
+    paths = [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(HERE, "emu_runtime.cpp")]
+    with ThreadPoolExecutor(max_workers=min(len(paths), os.cpu_count() or 4)) as ex:
+        objs = list(ex.map(_compile, paths))
+    r = subprocess.run([CXX, "-shared", "-fPIC", "-o", LIB + ".tmp"] + objs + ["-lpthread", "-lm"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"emulator link failed:\n{r.stdout[-4000:]}")
+    os.replace(LIB + ".tmp", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build())

@@ -1,0 +1,245 @@
+// Fiber scheduler of the wave64 emulator (test infrastructure; see emu_runtime.h).
+#include "emu_runtime.h"
+
+#include <stdio.h>
+#include <sys/mman.h>
+
+#include <vector>
+
+namespace emu {
+
+thread_local Lane* cur = nullptr;
+
+namespace {
+
+constexpr size_t kStack = 512 << 10;
+constexpr size_t kLdsBytes = 160 << 10;
+constexpr int kMaxThreads = 1024;
+
+struct Fiber {
+    Lane lane;
+    void* sp;
+    bool done;
+};
+
+struct WaveState {
+    int live, arrived;
+    unsigned gen;
+    alignas(64) char buf[2][64][256];
+};
+
+struct Group {
+    std::vector<Fiber> fibers;
+    std::vector<WaveState> waves;
+    char* stacks = nullptr;
+    char* lds = nullptr;
+    int n = 0, live = 0, running = -1;
+    int bar_arrived = 0;
+    unsigned bar_gen = 0;
+    void* main_sp = nullptr;
+    const std::function<void()>* body = nullptr;
+    long idle = 0;  // consecutive yields without progress
+    bool failed = false;
+    char why[256];
+};
+
+Group g;
+hipError_t last_error = hipSuccess;
+
+extern "C" void emu_switch(void** save_sp, void* to_sp);
+asm(R"(
+    .text
+    .globl emu_switch
+    .type emu_switch,@function
+emu_switch:
+    pushq %rbp
+    pushq %rbx
+    pushq %r12
+    pushq %r13
+    pushq %r14
+    pushq %r15
+    movq %rsp, (%rdi)
+    movq %rsi, %rsp
+    popq %r15
+    popq %r14
+    popq %r13
+    popq %r12
+    popq %rbx
+    popq %rbp
+    ret
+)");
+
+void fail(const char* what)
+{
+    if (!g.failed) {
+        g.failed = true;
+        snprintf(g.why, sizeof(g.why), "%s (workgroup %u,%u,%u thread %u)", what, cur->bid.x, cur->bid.y, cur->bid.z, cur->tid.x);
+        fprintf(stderr, "emu: %s\n", g.why);
+    }
+}
+
+// run the next fiber that has not finished; back to the launcher when none is left
+void schedule()
+{
+    const int from = g.running;
+    void** save = from >= 0 ? &g.fibers[from].sp : &g.main_sp;
+    if (g.live == 0 || g.failed) {
+        g.running = -1;
+        cur = nullptr;
+        if (from >= 0) emu_switch(save, g.main_sp);
+        return;
+    }
+    int next = from;
+    do {
+        next = (next + 1) % g.n;
+    } while (g.fibers[next].done);
+    if (next == from) return;
+    g.running = next;
+    cur = &g.fibers[next].lane;
+    emu_switch(save, g.fibers[next].sp);
+}
+
+void yield_waiting()
+{
+    // every live fiber waiting and nobody making progress for several rounds: the kernel deadlocked (lanes of a wave took
+    // different paths to a cross-lane instruction, or a barrier that not every wave reaches)
+    if (++g.idle > 8L * g.n + 64) fail("deadlock: a rendezvous that not every live lane reaches");
+    schedule();
+}
+
+void fiber_exit()
+{
+    Fiber& f = g.fibers[g.running];
+    f.done = true;
+    --g.live;
+    WaveState& w = g.waves[f.lane.wave];
+    --w.live;
+    if (w.arrived > 0 && w.arrived >= w.live) fail("a lane ended while other lanes of its wave wait in a cross-lane instruction");
+    if (g.bar_arrived > 0 && g.bar_arrived >= g.live) {  // the hardware barrier does not wait for ended waves
+        g.bar_arrived = 0;
+        ++g.bar_gen;
+    }
+    g.idle = 0;
+    schedule();
+    abort();  // a finished fiber is never resumed
+}
+
+void fiber_main()
+{
+    (*g.body)();
+    fiber_exit();
+}
+
+}  // namespace
+
+hipError_t take_error()
+{
+    const hipError_t e = last_error;
+    last_error = hipSuccess;
+    return e;
+}
+
+char* dynamic_lds() { return g.lds; }
+
+void barrier()
+{
+    const unsigned gen = g.bar_gen;
+    if (++g.bar_arrived >= g.live) {
+        g.bar_arrived = 0;
+        ++g.bar_gen;
+        g.idle = 0;
+        return;
+    }
+    while (g.bar_gen == gen && !g.failed) yield_waiting();
+}
+
+const char* exchange(const void* mine, size_t n)
+{
+    WaveState& w = g.waves[cur->wave];
+    const unsigned gen = w.gen;
+    char(*slots)[256] = w.buf[gen & 1];
+    memcpy(slots[cur->lane], mine, n);
+    if (++w.arrived >= w.live) {
+        if (w.live != 64 && w.live != (int)(g.n - cur->wave * 64))
+            fail("cross-lane instruction with lanes of the wave already ended");
+        w.arrived = 0;
+        ++w.gen;
+        g.idle = 0;
+    } else {
+        while (w.gen == gen && !g.failed) yield_waiting();
+    }
+    return &slots[0][0];
+}
+
+int readfirstlane(int x) { return lane_value<int>(exchange(&x, 4), 0); }
+
+uint64_t ballot(bool p)
+{
+    const char c = p ? 1 : 0;
+    const char* all = exchange(&c, 1);
+    const int lanes = g.n - cur->wave * 64 < 64 ? g.n - cur->wave * 64 : 64;
+    uint64_t m = 0;
+    for (int i = 0; i < lanes; ++i) m |= (uint64_t)(all[(size_t)i * 256] != 0) << i;
+    return m;
+}
+
+void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>& body)
+{
+    const int n = (int)(block.x * block.y * block.z);
+    if (n <= 0 || n > kMaxThreads || lds_bytes > kLdsBytes) {
+        last_error = hipErrorInvalidValue;
+        return;
+    }
+    if (!g.stacks) {
+        g.stacks = (char*)mmap(nullptr, kStack * kMaxThreads, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+        g.lds = (char*)mmap(nullptr, kLdsBytes, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_32BIT, -1, 0);
+        if (g.stacks == MAP_FAILED || g.lds == MAP_FAILED) {
+            fprintf(stderr, "emu: cannot map fiber stacks / LDS\n");
+            abort();
+        }
+    }
+    g.fibers.resize(n);
+    g.waves.resize((n + 63) / 64);
+    g.n = n;
+    g.body = &body;
+    g.failed = false;
+    for (unsigned bz = 0; bz < grid.z && !g.failed; ++bz)
+        for (unsigned by = 0; by < grid.y && !g.failed; ++by)
+            for (unsigned bx = 0; bx < grid.x && !g.failed; ++bx) {
+                // LDS content of the previous workgroup is poison, as on the hardware where it is whatever was there
+                memset(g.lds, 0xff, lds_bytes ? lds_bytes : 64);
+                for (auto& w : g.waves) {
+                    w.live = 0;
+                    w.arrived = 0;
+                    w.gen = 0;
+                }
+                for (int t = 0; t < n; ++t) {
+                    Fiber& f = g.fibers[t];
+                    f.lane.tid = dim3(t % block.x, (t / block.x) % block.y, t / (block.x * block.y));
+                    f.lane.bid = dim3(bx, by, bz);
+                    f.lane.bdim = block;
+                    f.lane.gdim = grid;
+                    f.lane.lane = t & 63;
+                    f.lane.wave = t >> 6;
+                    f.done = false;
+                    ++g.waves[t >> 6].live;
+                    // initial frame: six callee-saved registers, then the entry point as return address; the stack
+                    // pointer is 8 modulo 16 when fiber_main starts, as after a call
+                    uintptr_t top = (uintptr_t)(g.stacks + (size_t)(t + 1) * kStack) & ~(uintptr_t)15;
+                    void** sp = (void**)(top - 8);
+                    *--sp = (void*)&fiber_main;
+                    for (int r = 0; r < 6; ++r) *--sp = nullptr;
+                    f.sp = sp;
+                }
+                g.live = n;
+                g.bar_arrived = 0;
+                g.bar_gen = 0;
+                g.idle = 0;
+                g.running = -1;
+                schedule();  // returns when every fiber has finished (or the kernel failed)
+            }
+    if (g.failed) last_error = hipErrorLaunchFailure;
+    g.body = nullptr;
+}
+
+}  // namespace emu

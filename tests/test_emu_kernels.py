@@ -1,0 +1,69 @@
+"""The kernel sources on a wave64 emulator, on the CPU: the GPU parity tests, re-run without a GPU.
+
+tests/emu/ compiles the UNCHANGED kernel sources of flashck_amd/csrc (and the C ABI in front of them) as host C++ on top
+of an emulator that runs every thread of a workgroup as a fiber and makes every cross-lane instruction (MFMA, lane
+permutes, readlane, ballot, transposing LDS read) and every barrier a rendezvous.  This module takes the test functions
+of the GPU test modules as they are and runs them against that build, with CPU tensors: the same inputs, the same
+oracle, the same tolerances.  It shows the kernels' indexing, swizzles, masks, table lookups and arithmetic to be
+right; it cannot show timing-dependent faults (a missing wait on an asynchronous load, a race between waves) and it
+says nothing about speed.  The emulator is test infrastructure: nothing outside tests/ loads it, and the operators
+still refuse to run without the HIP library.
+
+By default only the cases listed in tests/emu/quick_cases.txt run (about two minutes in one process); FCK_EMU_FULL=1
+runs every collected case (`FCK_EMU_FULL=1 python -m pytest tests/test_emu_kernels.py -n 8`: several minutes on 8 cores).
+Tests that need a real device (graph capture, the C++ header program, timing) are left out by name.
+"""
+import ctypes
+import importlib
+import os
+import sys
+
+import pytest
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "emu"))
+
+GPU_MODULES = ["test_gpu_decode", "test_gpu_combine", "test_gpu_appendkv", "test_gpu_prefill", "test_gpu_prefill_grid",
+               "test_gpu_score_mods", "test_gpu_head_dims", "test_gpu_step", "test_gpu_validate", "test_zz_no_alloc"]
+# need a real device: HIP graph capture, event timing of the tuner, device-property queries
+NEEDS_DEVICE = {"test_decode_captured_in_a_graph", "test_tuner_picks_and_caches", "test_tuner_records_kernel_variant"}
+
+_mods = [importlib.import_module(m) for m in GPU_MODULES]
+for _m in _mods:
+    for _name in dir(_m):
+        _fn = getattr(_m, _name)
+        if _name.startswith("test_") and callable(_fn) and _name not in NEEDS_DEVICE:
+            globals()[f"test_emu_{_m.__name__[5:]}__{_name[5:]}"] = _fn
+
+
+def _cpu(x, device="cpu"):
+    """stand-in for helpers.dev: a private copy on the CPU (kernels write in place, as they do to device copies)"""
+    return x.clone() if isinstance(x, torch.Tensor) else x
+
+
+@pytest.fixture(scope="module")
+def fmha():
+    """flashck_amd.ops.fmha bound to the emulator build for the duration of this module."""
+    import build_emu
+    from flashck_amd import _lib
+    from flashck_amd.ops import fmha as ops
+    from flashck_amd.ops.fmha import fmha as F
+    path = build_emu.build()
+    lib = ctypes.CDLL(path)
+    for name, (res, args) in _lib.SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    saved = dict(lib=_lib._lib, req=F._REQUIRE_GPU_TENSORS, stream=F._stream, sync=torch.cuda.synchronize,
+                 devs=[(m, m.dev) for m in _mods if hasattr(m, "dev")])
+    _lib._lib, F._REQUIRE_GPU_TENSORS, F._stream = lib, False, (lambda: None)
+    torch.cuda.synchronize = lambda *a, **k: None
+    for m, _ in saved["devs"]:
+        m.dev = _cpu
+    try:
+        yield ops
+    finally:
+        _lib._lib, F._REQUIRE_GPU_TENSORS, F._stream = saved["lib"], saved["req"], saved["stream"]
+        torch.cuda.synchronize = saved["sync"]
+        for m, d in saved["devs"]:
+            m.dev = d

@@ -175,3 +175,21 @@ def test_caller_supplied_buffers_are_validated(host_ops):
     kn = torch.zeros(B, 1, Hk, D, dtype=T)
     with pytest.raises(ValueError, match="do not match knew"):
         fmha.fmha_fwd_appendkv(None, kc, torch.zeros(8, P, Hk, 32, dtype=T), kn, kn, sl, block_table=bt)
+
+
+def test_validate_paged_arguments_are_checked_before_any_launch():
+    """fck_fmha_validate_paged: argument errors come back as a status, without a GPU."""
+    import ctypes
+    lib = _lib.load()
+    buf = (ctypes.c_int32 * 8)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    rc = lib.fck_fmha_validate_paged(p, p, 2, None, None, None, 0, 4, 16, p, None)          # batch 0
+    assert rc == -1 and b"positive" in lib.fck_last_error()
+    rc = lib.fck_fmha_validate_paged(p, p, 2, p, p, None, 1, 4, 16, p, None)                # table and list
+    assert rc == -1 and b"either" in lib.fck_last_error()
+    rc = lib.fck_fmha_validate_paged(None, None, 0, None, None, None, 1, 4, 16, p, None)    # neither
+    assert rc == -1 and b"either" in lib.fck_last_error()
+    rc = lib.fck_fmha_validate_paged(None, p, 2, None, None, None, 1, 4, 16, p, None)       # table without lengths
+    assert rc == -1 and b"seqlen_k" in lib.fck_last_error()
+    rc = lib.fck_fmha_validate_paged(p, p, 2, None, None, None, 1, 4, 16, None, None)       # no counters
+    assert rc == -1 and b"error_counts" in lib.fck_last_error()

@@ -178,3 +178,39 @@ def test_tuner_records_the_kernel_variant_with_the_split_count(tmp_path):
     c.insert(tuning.SPLITKV, tuning.splitkv_problem(*args), rec)
     assert tuning.choose_splitkv(lambda: 7, *args, cache=c) == (4, 1)
     assert tuning.choose_splitkv(lambda: 7, 8, 16, 4, 1, 2048, 128, 64, "bf16", cache=c) == (7, 0)   # another class: heuristic
+
+
+def test_cached_variant_is_only_a_hint():
+    """The tuning key buckets the query count and does not hold v_head_dim, so a record for one call can be served to a
+    call the recorded kernel variant cannot take; the Python layer re-checks the variant's preconditions."""
+    from flashck_amd.ops.fmha import fmha as F
+    assert F._usable_variant(2, 40, 8, 3, 128, 128) == 2     # 15 packed rows: head pairs fit
+    assert F._usable_variant(2, 40, 8, 4, 128, 128) == 0     # same query bucket, 20 packed rows: back to the library's choice
+    assert F._usable_variant(2, 32, 8, 1, 128, 64) == 0      # qk_head_dim != v_head_dim
+    assert F._usable_variant(2, 32, 8, 1, 256, 256) == 0     # head pairs exist for 64 and 128
+    assert F._usable_variant(2, 21, 7, 1, 128, 128) == 0     # odd number of KV heads
+    assert F._usable_variant(2, 32, 8, 1, 128, 128, plain=False) == 0   # score modifier / fp8 cache
+    assert F._usable_variant(1, 21, 7, 9, 256, 64) == 1      # one head per workgroup fits every call
+    assert F._usable_variant(7, 32, 8, 1, 128, 128) == 0     # nonsense in the cache
+
+
+def test_decode_step_drops_a_cached_variant_it_cannot_take(monkeypatch, tmp_path):
+    """fmha_decode_step with num_splits = 0 and a cache record (3 splits, head pairs) made with 3 new tokens: a step with
+    4 new tokens falls into the same class but packs 20 query rows per KV head; it must run with variant 0."""
+    import torch
+    from flashck_amd.ops.fmha import fmha as F
+    c = tuning.TuningCache(str(tmp_path), ENV)
+    flags.set_flag_value("FC_TUNING_MODE", "1")
+    c.insert(tuning.SPLITKV, tuning.splitkv_problem(2, 40, 8, 3, 256, 128, 128, "bf16"), dict(num_splits=3, variant=2))
+    monkeypatch.setattr(tuning, "default_cache", lambda: c)
+    seen = []
+    monkeypatch.setattr(F, "_REQUIRE_GPU_TENSORS", False)
+    monkeypatch.setattr(F, "fmha_fwd_appendkv", lambda *a, **k: None)
+    monkeypatch.setattr(F, "fmha_fwd_splitkv", lambda *a, **k: seen.append((a[3], k["decode_variant"])) or (k["o_acc"], k["lse_acc"]))
+    monkeypatch.setattr(F, "fmha_fwd_splitkv_combine", lambda lse, o, dt, **k: torch.empty(0))
+    for n, want in ((3, 2), (4, 0)):
+        q = torch.zeros(2, n, 40, 128, dtype=torch.bfloat16)
+        kn = torch.zeros(2, n, 8, 128, dtype=torch.bfloat16)
+        kc = torch.zeros(4, 128, 8, 128, dtype=torch.bfloat16)
+        F.fmha_decode_step(q, kn, kn, kc, kc, torch.tensor([5, 9], dtype=torch.int32), torch.tensor([[0, 1], [2, 3]], dtype=torch.int32))
+        assert seen[-1] == (3, want), (n, seen[-1])
