@@ -25,7 +25,7 @@ def _compile(path):
     obj = os.path.join(OBJ, os.path.splitext(os.path.basename(path))[0] + ".o")
     if os.path.exists(obj) and os.path.getmtime(obj) > max(
             os.path.getmtime(os.path.join(d, f)) for d in (CSRC, HERE, os.path.join(HERE, "include"), os.path.join(ROOT, "include", "flashck", "fmha"))
-            for f in os.listdir(d) if os.path.isfile(os.path.join(d, f))):
+            for f in os.listdir(d) if f.endswith((".hip", ".hpp", ".h", ".cpp"))):
         return obj
     r = subprocess.run([CXX] + FLAGS + ["-c", path, "-o", obj], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
@@ -38,11 +38,24 @@ def build():
     paths = [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(HERE, "emu_runtime.cpp")]
     with ThreadPoolExecutor(max_workers=min(len(paths), os.cpu_count() or 4)) as ex:
         objs = list(ex.map(_compile, paths))
+    if os.path.exists(LIB) and os.path.getmtime(LIB) >= max(os.path.getmtime(o) for o in objs):
+        return LIB
     r = subprocess.run([CXX, "-shared", "-fPIC", "-o", LIB + ".tmp"] + objs + ["-lpthread", "-lm"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"emulator link failed:\n{r.stdout[-4000:]}")
     os.replace(LIB + ".tmp", LIB)
     return LIB
+
+
+def build_pybind():
+    """flash_ck/csrc/pybind.cpp bound to the emulator library: module `flash_ck_emu` in this directory."""
+    import sysconfig
+    from flash_ck import build as fb
+    out = os.path.join(HERE, "flash_ck_emu" + sysconfig.get_config_var("EXT_SUFFIX"))
+    src = os.path.join(ROOT, "flash_ck", "csrc", "pybind.cpp")
+    if os.path.exists(out) and os.path.getmtime(out) > max(os.path.getmtime(src), os.path.getmtime(LIB)):
+        return out
+    return fb.build(name="flash_ck_emu", out=out, kernel_lib=LIB, extra=["-DFLASH_CK_HOST_TENSORS"])
 
 
 if __name__ == "__main__":

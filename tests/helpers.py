@@ -5,6 +5,10 @@ import torch
 ATOL = {torch.float16: 1e-2, torch.bfloat16: 2e-2}
 
 
+# where the parity tests put their tensors (the emulator run of these tests sets it to "cpu")
+DEVICE = "cuda"
+
+
 def dev(x, device="cuda"):
     if isinstance(x, torch.Tensor):
         return x.to(device)

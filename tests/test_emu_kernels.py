@@ -25,9 +25,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(HERE, "emu"))
 
 GPU_MODULES = ["test_gpu_decode", "test_gpu_combine", "test_gpu_appendkv", "test_gpu_prefill", "test_gpu_prefill_grid",
-               "test_gpu_score_mods", "test_gpu_head_dims", "test_gpu_step", "test_gpu_validate", "test_zz_no_alloc"]
-# need a real device: HIP graph capture, event timing of the tuner, device-property queries
-NEEDS_DEVICE = {"test_decode_captured_in_a_graph", "test_tuner_picks_and_caches", "test_tuner_records_kernel_variant"}
+               "test_gpu_score_mods", "test_gpu_head_dims", "test_gpu_step", "test_gpu_validate", "test_zy_flash_ck_module",
+               "test_zz_no_alloc"]
+# need a real device: HIP graph capture
+NEEDS_DEVICE = {"test_decode_captured_in_a_graph"}
 
 _mods = [importlib.import_module(m) for m in GPU_MODULES]
 for _m in _mods:
@@ -35,6 +36,7 @@ for _m in _mods:
         _fn = getattr(_m, _name)
         if _name.startswith("test_") and callable(_fn) and _name not in NEEDS_DEVICE:
             globals()[f"test_emu_{_m.__name__[5:]}__{_name[5:]}"] = _fn
+del _fn
 
 
 def _cpu(x, device="cpu"):
@@ -42,28 +44,66 @@ def _cpu(x, device="cpu"):
     return x.clone() if isinstance(x, torch.Tensor) else x
 
 
-@pytest.fixture(scope="module")
-def fmha():
-    """flashck_amd.ops.fmha bound to the emulator build for the duration of this module."""
+def _wall_timer(fn, cold, repeats):
+    """stand-in for tuning.gpu_timer (events on a stream): wall clock around one call; which candidate wins is not
+    what these tests check"""
+    import time
+    t0 = time.perf_counter()
+    fn()
+    return time.perf_counter() - t0
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _emulator_bound():
+    """flashck_amd.ops.fmha (and flashck_amd._lib.load) bound to the emulator build for the duration of this module."""
     import build_emu
+    import helpers
     from flashck_amd import _lib
     from flashck_amd.ops import fmha as ops
     from flashck_amd.ops.fmha import fmha as F
+    from flashck_amd.utils import tuning
     path = build_emu.build()
     lib = ctypes.CDLL(path)
     for name, (res, args) in _lib.SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = res, args
-    saved = dict(lib=_lib._lib, req=F._REQUIRE_GPU_TENSORS, stream=F._stream, sync=torch.cuda.synchronize,
-                 devs=[(m, m.dev) for m in _mods if hasattr(m, "dev")])
+    saved = dict(lib=_lib._lib, req=F._REQUIRE_GPU_TENSORS, stream=F._stream, sync=torch.cuda.synchronize, device=helpers.DEVICE,
+                 timer=tuning.gpu_timer, devs=[(m, m.dev) for m in _mods if hasattr(m, "dev")],
+                 streams=[(m, m._stream) for m in _mods if hasattr(m, "_stream")])
     _lib._lib, F._REQUIRE_GPU_TENSORS, F._stream = lib, False, (lambda: None)
     torch.cuda.synchronize = lambda *a, **k: None
+    helpers.DEVICE = "cpu"
+    tuning.gpu_timer = _wall_timer
     for m, _ in saved["devs"]:
         m.dev = _cpu
+    for m, _ in saved["streams"]:
+        m._stream = lambda: None
     try:
         yield ops
     finally:
         _lib._lib, F._REQUIRE_GPU_TENSORS, F._stream = saved["lib"], saved["req"], saved["stream"]
         torch.cuda.synchronize = saved["sync"]
+        helpers.DEVICE = saved["device"]
+        tuning.gpu_timer = saved["timer"]
         for m, d in saved["devs"]:
             m.dev = d
+        for m, f in saved["streams"]:
+            m._stream = f
+
+
+@pytest.fixture(scope="module")
+def fmha(_emulator_bound):
+    return _emulator_bound
+
+
+@pytest.fixture(scope="module")
+def fck(fmha):
+    """The glue of the compiled `flash_ck` module (flash_ck/csrc/pybind.cpp), built against the emulator library with
+    host tensors allowed, next to the emulator-bound functional API."""
+    import types
+    import build_emu
+    build_emu.build_pybind()
+    import flash_ck_emu
+    ns = types.SimpleNamespace(**{n: getattr(flash_ck_emu, n) for n in dir(flash_ck_emu) if n.startswith("fmha_")})
+    ns.ops = types.SimpleNamespace(fmha=fmha)
+    return ns

@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from flashck_amd import _lib, generators as gen
+import helpers
 from helpers import ATOL, assert_close, assert_lse_close, dev
 
 pytestmark = pytest.mark.gpu
@@ -170,11 +171,11 @@ def test_modifier_arguments_are_validated(fmha):
     with pytest.raises(TypeError):
         fmha.fmha_fwd(q, k, v, bias=dev(gen.randn((1, 4, 4, 4), torch.bfloat16, g)))         # wrong dtype
     with pytest.raises(ValueError):
-        fmha.fmha_fwd(q, k, v, alibi_slopes=torch.ones(3, dtype=torch.float32, device="cuda"))  # wrong head count
+        fmha.fmha_fwd(q, k, v, alibi_slopes=torch.ones(3, dtype=torch.float32, device=helpers.DEVICE))  # wrong head count
     with pytest.raises(ValueError):
         fmha.fmha_fwd(q, k, v, logits_soft_cap=-1.0)
     with pytest.raises(NotImplementedError):                                                 # ALiBi has no diagonal for GENERIC
-        fmha.fmha_fwd(q, k, v, mask_type=3, window=(1, 1), alibi_slopes=torch.ones(4, dtype=torch.float32, device="cuda"))
+        fmha.fmha_fwd(q, k, v, mask_type=3, window=(1, 1), alibi_slopes=torch.ones(4, dtype=torch.float32, device=helpers.DEVICE))
     # a raw bias pointer without attributes is refused by the C ABI (nothing says what it holds)
     import ctypes
     lib = _lib.load()
@@ -239,7 +240,7 @@ def test_fp8_cache_is_refused_where_no_kernel_reads_it(fmha):
     lib = _lib.load()
     at = _lib.Attrs()
     at.size, at.kv_dtype = ctypes.sizeof(_lib.Attrs), 1
-    x = torch.zeros(1, 4, 4, 64, dtype=torch.float16, device="cuda")
+    x = torch.zeros(1, 4, 4, 64, dtype=torch.float16, device=helpers.DEVICE)
     rc = lib.fck_fmha_fwd_attrs(x.data_ptr(), x.data_ptr(), x.data_ptr(), None, x.data_ptr(), None, None, None, 1, 4, 4, 4, 4, 64, 64,
                                 4, 0.125, -1, -1, 0, 3, ctypes.byref(at), None)
     assert rc == -2 and b"split-KV entry point only" in lib.fck_last_error()

@@ -3,6 +3,7 @@ import pytest
 import torch
 
 from flashck_amd import generators as gen
+import helpers
 from helpers import assert_bits_equal, assert_close, dev
 
 pytestmark = pytest.mark.gpu
@@ -172,9 +173,9 @@ def test_decode_captured_in_a_graph(fmha, orc, fused):
     kc, vc, bt = dev(kv["k_cache"]), dev(kv["v_cache"]), dev(kv["block_table"])
     sl = dev(kv["seqlen_k"].clone())           # advanced in place by the captured graph's caller between replays
     sl_after = torch.empty_like(sl)
-    q, knew, vnew = (torch.empty(B, 1, h, d, dtype=torch.bfloat16, device="cuda") for h in (hq, hk, hk))
-    out = torch.empty(B, 1, hq, d, dtype=torch.bfloat16, device="cuda")
-    ws = fmha.splitkv_workspace(B, hq, 1, d, 3, "cuda")
+    q, knew, vnew = (torch.empty(B, 1, h, d, dtype=torch.bfloat16, device=helpers.DEVICE) for h in (hq, hk, hk))
+    out = torch.empty(B, 1, hq, d, dtype=torch.bfloat16, device=helpers.DEVICE)
+    ws = fmha.splitkv_workspace(B, hq, 1, d, 3, helpers.DEVICE)
     dcos, dsin = dev(cos), dev(sin)
 
     def enqueue():

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from flashck_amd import _lib, generators as gen
+import helpers
 from helpers import assert_bits_equal, assert_close, dev
 
 pytestmark = pytest.mark.gpu
@@ -33,14 +34,14 @@ def _run_both(lib, kv, q, ns, mask_type=0, window=(-1, -1), cu=None, max_sq=0):
     qd, kc, vc = dev(q), dev(kv["k_cache"]), dev(kv["v_cache"])
     sl, bt, cud = dev(kv["seqlen_k"]), dev(kv["block_table"]), dev(cu)
     scale = 1.0 / math.sqrt(D)
-    o_fused = torch.full(q.shape, float("nan"), dtype=q.dtype, device="cuda")
+    o_fused = torch.full(q.shape, float("nan"), dtype=q.dtype, device=helpers.DEVICE)
     rc = lib.fck_fmha_fwd_splitkv_fused(_vp(qd), _vp(kc), _vp(vc), None, _vp(o_fused), _vp(cud), None, _vp(sl), _vp(bt), None,
                                         B, sq, 0, Hq, Hk, D, D, max_sq, ns, bt.numel(), page, scale, window[0], window[1],
                                         mask_type, dt, _stream())
     assert rc == 0, lib.fck_last_error().decode()
-    o_acc = torch.empty(bs, Hq, ns, sq, D, dtype=torch.float32, device="cuda")
-    lse_acc = torch.empty(bs, Hq, ns, sq, dtype=torch.float32, device="cuda")
-    o_ref = torch.full(q.shape, float("nan"), dtype=q.dtype, device="cuda")
+    o_acc = torch.empty(bs, Hq, ns, sq, D, dtype=torch.float32, device=helpers.DEVICE)
+    lse_acc = torch.empty(bs, Hq, ns, sq, dtype=torch.float32, device=helpers.DEVICE)
+    o_ref = torch.full(q.shape, float("nan"), dtype=q.dtype, device=helpers.DEVICE)
     rc = lib.fck_fmha_fwd_splitkv(_vp(qd), _vp(kc), _vp(vc), None, _vp(lse_acc), _vp(o_acc), _vp(cud), None, _vp(sl), _vp(bt),
                                   None, B, sq, 0, Hq, Hk, D, D, max_sq, ns, bt.numel(), page, scale, window[0], window[1],
                                   mask_type, dt, _stream())
@@ -89,8 +90,8 @@ def test_fused_library_chosen_split_count(orc):
 
 def test_fused_rejects_what_does_not_fit():
     lib = _lib.load()
-    x = torch.zeros(64, dtype=torch.bfloat16, device="cuda")
-    i = torch.zeros(64, dtype=torch.int32, device="cuda")
+    x = torch.zeros(64, dtype=torch.bfloat16, device=helpers.DEVICE)
+    i = torch.zeros(64, dtype=torch.int32, device=helpers.DEVICE)
     # 64 sequences x 64 heads x 128 splits x 129 floats > 4 Mi floats
     rc = lib.fck_fmha_fwd_splitkv_fused(_vp(x), _vp(x), _vp(x), None, _vp(x), None, None, _vp(i), _vp(i), None, 64, 1, 0, 64, 8,
                                         128, 128, 1, 128, 64 * 4, 128, 0.1, -1, -1, 0, 4, _stream())
