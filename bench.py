@@ -22,7 +22,16 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
 
 COUNTER_FILE = os.path.join(ROOT, "profiles", "splitkv_decode_cfg3.md")
-DECODE_SOURCE = os.path.join(ROOT, "flashck_amd", "csrc", "splitkv_decode.hip")
+# every source file that goes into the device code of the split-KV kernel
+DECODE_SOURCES = [os.path.join(ROOT, "flashck_amd", "csrc", f) for f in ("splitkv_decode.hip", "common.hpp", "kernels.hpp", "gfx950_ops.hpp")]
+
+
+def decode_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for path in DECODE_SOURCES:
+        h.update(open(path, "rb").read())
+    return h.hexdigest()
 
 
 def measured_traffic(kernel):
@@ -31,13 +40,13 @@ def measured_traffic(kernel):
     The figure is not measured by this run: it comes from the `counters` line of profiles/splitkv_decode_cfg3.md (two
     `rocprofv3 --pmc` runs of this script, FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same
     counter reads for a plain device copy of known size).  It is only reported while it still describes the code that
-    runs: same kernel variant and same source file as when the counters were read.
+    runs: same kernel variant and same source files (the kernel and the headers it is built from) as when the
+    counters were read.
     """
-    import hashlib
     import re
     try:
         text = open(COUNTER_FILE).read()
-        sha = hashlib.sha256(open(DECODE_SOURCE, "rb").read()).hexdigest()
+        sha = decode_source_hash()
     except OSError:
         return None
     m = re.search(r'counters kernel="([^"]+)" source_sha256=([0-9a-f]+) fetch_kib=([0-9.]+) write_kib=([0-9.]+) '
@@ -57,15 +66,15 @@ def parse():
     ap.add_argument("--copies", type=int, default=4, help="KV pool copies rotated between steps")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--kv-len", type=int, default=32768, help="KV length of the split-KV workload (study runs only)")
-    ap.add_argument("--no-shuffle", action="store_true", help="identity page order (study runs only)")
-    ap.add_argument("--num-splits", type=int, default=8, help="split count of the split-KV workload (study runs only)")
     ap.add_argument("--paged-splits", type=int, default=0, help="split count of the paged-decode workload (0: the library's heuristic)")
     ap.add_argument("--kv-fp8", action="store_true", help="split-KV workload with the cache stored as fp8 (e4m3, static scales)")
     ap.add_argument("--decode-path", default="two-launch", choices=["two-launch", "fused"],
                     help="two-launch: split-KV + combine kernels with a caller-owned workspace; fused: one launch "
                          "(--num-splits 0 lets the library choose the key ranges)")
-    return ap.parse_args()
+    args = ap.parse_args()
+    # the split-KV workload as BASELINE config 3 states it
+    args.kv_len, args.num_splits, args.no_shuffle = 32768, 8, False
+    return args
 
 
 def time_steps(fn, steps, warmup, torch, kernel_events=False):

@@ -17,7 +17,8 @@ class Attrs(ctypes.Structure):
     _fields_ = [("size", ctypes.c_uint32), ("bias_type", ctypes.c_int32), ("bias", ctypes.c_void_p),
                 ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64),
                 ("logits_soft_cap", ctypes.c_float), ("kv_dtype", ctypes.c_int32), ("k_descale", ctypes.c_float),
-                ("v_descale", ctypes.c_float), ("decode_variant", ctypes.c_int32)]
+                ("v_descale", ctypes.c_float), ("decode_variant", ctypes.c_int32), ("prefill_variant", ctypes.c_int32),
+                ("bias_cols", ctypes.c_int64)]
 
 
 _ap = ctypes.POINTER(Attrs)
@@ -39,6 +40,8 @@ SIGNATURES = {
     "fck_fmha_fwd_splitkv_combine": (ctypes.c_int, [_vp] * 4 + [_i64] * 6 + [_i32, _vp]),
     "fck_fmha_fwd_appendkv": (ctypes.c_int, [_vp] * 7 + [_i64, _vp, _vp, _i64, _i32, _i32, _vp, _i64, _i64, _vp]
                               + [_i64] * 6 + [_i32, _vp]),
+    "fck_fmha_fwd_appendkv_attrs": (ctypes.c_int, [_vp] * 7 + [_i64, _vp, _vp, _i64, _i32, _i32, _vp, _i64, _i64, _vp]
+                                    + [_i64] * 6 + [_i32, _ap, _vp]),
     "fck_fmha_batch_prefill": (ctypes.c_int, [_vp] * 8 + [_i64] * 8 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_fwd_pagedkv": (ctypes.c_int, [_vp] * 7 + [_i64] * 9 + [_f32, _i64, _i64, _u32, _i32, _vp]),
     "fck_fmha_num_splits_heuristic": (ctypes.c_int, [_i64] * 7),

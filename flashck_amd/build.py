@@ -16,7 +16,7 @@ OBJ = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libflashck_fmha.so")
 
 SOURCES = ["fmha_api.cpp", "splitkv_decode.hip", "splitkv_combine.hip", "appendkv_rope.hip", "prefill.hip",
-           "prefill_pingpong.hip", "prefill_dma.hip", "validate.hip"]
+           "prefill_pingpong.hip", "prefill_dma.hip", "validate.hip", "appendkv_fp8.hip"]
 
 FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "--offload-arch=gfx950", "-fno-gpu-rdc",
@@ -34,8 +34,15 @@ def hipcc():
     return exe
 
 
-def _compile(src, extra):
+def _newest_header():
+    dirs = (CSRC, os.path.join(ROOT, "include", "flashck", "fmha"))
+    return max(os.path.getmtime(os.path.join(d, f)) for d in dirs for f in os.listdir(d) if f.endswith((".hpp", ".h")))
+
+
+def _compile(src, extra, incremental=False):
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(os.path.join(CSRC, src)), _newest_header()):
+        return obj, ""
     cmd = [hipcc(), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS + extra
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
@@ -44,10 +51,12 @@ def _compile(src, extra):
     return obj, out
 
 
-def build(verbose=False, extra_flags=()):
+def build(verbose=False, extra_flags=(), incremental=False):
+    """incremental: translation units whose object file is newer than the source and every header are not recompiled
+    (a development convenience; the default compiles everything)."""
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 4)) as ex:
-        results = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
+        results = list(ex.map(lambda s: _compile(s, list(extra_flags), incremental), SOURCES))
     objs = [o for o, _ in results]
     if verbose:
         for _, out in results:
@@ -85,4 +94,5 @@ def build_header_test():
 
 
 if __name__ == "__main__":
-    print(build(verbose=True, extra_flags=sys.argv[1:]))
+    flags = [a for a in sys.argv[1:] if a != "--incremental"]
+    print(build(verbose=True, extra_flags=flags, incremental="--incremental" in sys.argv[1:]))

@@ -131,6 +131,24 @@ __device__ __forceinline__ float quad16_sum(float x)
     return pair32_sum(a + b);
 }
 
+// 8 e4m3 bytes (the two low dwords of v) widened to 8 elements of T; exact, every e4m3 value is a T value
+template <typename T>
+__device__ __forceinline__ u32x4_t fp8x8_to_t(u32x4_t v)
+{
+    const f32x2_t a0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[0], false), a1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[0], true);
+    const f32x2_t a2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[1], false), a3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[1], true);
+    return u32x4_t{T::pack2(a0[0], a0[1]), T::pack2(a1[0], a1[1]), T::pack2(a2[0], a2[1]), T::pack2(a3[0], a3[1])};
+}
+
+// fp32 -> e4m3 byte (OCP encoding): round to nearest even; finite values saturate at +-448, NaN and infinities are left
+// to the conversion instruction (as ck_tile converts: ck_tile/core/numeric/float8.hpp:600-662)
+__device__ __forceinline__ uint32_t f32_to_fp8_sat(float x)
+{
+    const bool finite = (__builtin_bit_cast(uint32_t, x) & 0x7f800000u) != 0x7f800000u;
+    const float c = finite ? fminf(fmaxf(x, -448.f), 448.f) : x;
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xffu;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
@@ -240,6 +258,7 @@ __host__ __device__ inline int32_t mask_hi(const MaskYX& m, int32_t i, int32_t s
 struct ScoreMod {
     const void* bias;
     int64_t batch_stride, head_stride, row_stride;
+    int64_t cols;       // elementwise: columns of a bias row (0: not stated)
     int32_t bias_type;  // 0 none, 1 elementwise, 2 ALiBi
     float soft_cap;     // > 0: on
     float scale;        // the softmax scale in natural units (the soft cap is not linear, so it cannot be folded)
@@ -273,7 +292,7 @@ struct RowMod {
     float slope;               // ALiBi: signed slope (positive for VERTICAL, negative otherwise)
     int32_t zero;              // ALiBi: column of distance 0 (unused for VERTICAL)
     int32_t mode;
-    int32_t last_key;          // bias reads are clamped to the row's last key
+    int32_t last_key;          // bias reads are clamped to the row's last key and to the last column of the bias
     float scale, cap, cap_rcp;
     int32_t bias_type;
 
@@ -285,6 +304,7 @@ struct RowMod {
         cap = m.soft_cap;
         cap_rcp = m.soft_cap > 0.f ? 1.f / m.soft_cap : 0.f;
         last_key = sk - 1;
+        if (m.cols > 0 && m.cols - 1 < last_key) last_key = (int32_t)(m.cols - 1);
         bias_row = nullptr;
         slope = 0.f;
         zero = 0;

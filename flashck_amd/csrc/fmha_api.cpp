@@ -18,6 +18,17 @@ namespace {
 thread_local char g_err[512] = "";
 thread_local const char* g_kernel = "";  // kernel family of the calling thread's last launch
 
+// "splitkv_decode_kernel<uniform_page|row_lookup[,head_pairs][,kv_fp8][,score_mod][,padded_head_dim][,fused]>": the
+// variant the calling thread's last split-KV launch took
+void name_decode_kernel(bool uniform, int heads_per_workgroup, bool kv8, bool mod, bool padded, bool fused)
+{
+    thread_local char name[128];
+    snprintf(name, sizeof(name), "splitkv_decode_kernel<%s%s%s%s%s%s>", uniform ? "uniform_page" : "row_lookup",
+             heads_per_workgroup == 2 ? ",head_pairs" : "", kv8 ? ",kv_fp8" : "", mod && !padded ? ",score_mod" : "",
+             padded ? ",padded_head_dim" : "", fused ? ",fused" : "");
+    g_kernel = name;
+}
+
 int fail(int code, const char* fmt, ...)
 {
     va_list ap;
@@ -48,13 +59,26 @@ int kernel_dim(int64_t d, int64_t dv)
     return m <= 64 ? 64 : m <= 128 ? 128 : 256;
 }
 
-// Bias / ALiBi / soft cap of a call: `bias` is the positional pointer of the entry points that have one (else null).
-int no_kv_dtype(const fck_fmha_attrs* at)
+// fp8 K/V with static per-tensor scales for the prefill entry points (after fill_mod): the K scale multiplies every
+// score, the V scale the output
+int fill_kv8(fck::PrefillArgs& a, const fck_fmha_attrs* at, int64_t d, int64_t dv)
 {
-    if (at && at->size == sizeof(fck_fmha_attrs) && at->kv_dtype != 0)
-        return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: a K/V cache type other than q's is read by the split-KV entry point only", at->kv_dtype);
+    a.kv8 = 0;
+    a.v_descale = 1.f;
+    if (!at || at->kv_dtype == 0) return FCK_OK;
+    if (at->kv_dtype != FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: only 0 (same as q) and FLOAT8 (1)", at->kv_dtype);
+    const float kd = at->k_descale == 0.f ? 1.f : at->k_descale, vd = at->v_descale == 0.f ? 1.f : at->v_descale;
+    if (!(kd > 0.f) || !std::isfinite(kd) || !(vd > 0.f) || !std::isfinite(vd))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "k_descale and v_descale must be positive and finite (0: 1)");
+    if (d != dv || d != kernel_dim(d, dv)) return fail(FCK_ERR_UNSUPPORTED, "an fp8 K/V cache needs qk_head_dim = v_head_dim in {64, 128, 256}");
+    a.kv8 = 1;
+    a.scale_log2 *= kd;
+    a.mod.scale *= kd;
+    a.v_descale = vd;
     return FCK_OK;
 }
+
+// Bias / ALiBi / soft cap of a call: `bias` is the positional pointer of the entry points that have one (else null).
 
 int fill_mod(fck::ScoreMod& m, const void* bias, const fck_fmha_attrs* at, float scale, uint32_t mask_type, int64_t hq)
 {
@@ -79,6 +103,8 @@ int fill_mod(fck::ScoreMod& m, const void* bias, const fck_fmha_attrs* at, float
         if (reinterpret_cast<uintptr_t>(bias) & 1u) return fail(FCK_ERR_INVALID_ARGUMENT, "the bias must be 2-byte aligned");
         if (at->bias_row_stride <= 0 || at->bias_head_stride < 0 || at->bias_batch_stride < 0)
             return fail(FCK_ERR_INVALID_ARGUMENT, "elementwise bias: row stride must be positive, head and batch strides >= 0");
+        if (at->bias_cols < 0 || at->bias_cols > at->bias_row_stride)
+            return fail(FCK_ERR_INVALID_ARGUMENT, "elementwise bias: bias_cols %ld must be in [0, bias_row_stride %ld]", (long)at->bias_cols, (long)at->bias_row_stride);
         break;
     case FCK_BIAS_ALIBI:
         if (!bias) return fail(FCK_ERR_INVALID_ARGUMENT, "bias_type ALIBI needs the slopes pointer");
@@ -95,6 +121,7 @@ int fill_mod(fck::ScoreMod& m, const void* bias, const fck_fmha_attrs* at, float
     m.batch_stride = at->bias_batch_stride;
     m.head_stride = at->bias_type == FCK_BIAS_ELEMENTWISE ? at->bias_head_stride : 0;
     m.row_stride = at->bias_type == FCK_BIAS_ELEMENTWISE ? at->bias_row_stride : 0;
+    m.cols = at->bias_type == FCK_BIAS_ELEMENTWISE && at->bias_cols > 0 ? at->bias_cols : 0;
     m.soft_cap = at->logits_soft_cap;
     m.scale = scale;
     return FCK_OK;
@@ -297,15 +324,10 @@ int fck_fmha_fwd_splitkv_attrs(const void* q, const void* k, const void* v, cons
     if (!aligned16(o_acc)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_acc must be 16-byte aligned");
     a.o_acc = static_cast<float*>(o_acc);
     a.lse_acc = static_cast<float*>(lse_acc);
-    static const char* const names[8] = {
-        "splitkv_decode_kernel<row_lookup>",         "splitkv_decode_kernel<uniform_page>",
-        "splitkv_decode_kernel<row_lookup,score_mod>", "splitkv_decode_kernel<uniform_page,score_mod>",
-        "splitkv_decode_kernel<row_lookup,kv_fp8>",  "splitkv_decode_kernel<uniform_page,kv_fp8>",
-        "splitkv_decode_kernel<row_lookup,kv_fp8,score_mod>", "splitkv_decode_kernel<uniform_page,kv_fp8,score_mod>"};
-    g_kernel = names[(a.kv8 ? 4 : 0) + (a.mod.active() ? 2 : 0) + (uniform ? 1 : 0)];
-    if (d != dv || d != kernel_dim(d, dv)) g_kernel = uniform ? "splitkv_decode_kernel<uniform_page,padded_head_dim>" : "splitkv_decode_kernel<row_lookup,padded_head_dim>";
-    return launch_status(fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
-                         "FmhaFwdSplitKV launch");
+    int hpw = 1;
+    const hipError_t e = fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream), &hpw);
+    name_decode_kernel(uniform, hpw, a.kv8 != 0, a.mod.active(), d != dv || d != kernel_dim(d, dv), false);
+    return launch_status(e, "FmhaFwdSplitKV launch");
 }
 
 int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, const void* bias, void* o,
@@ -351,9 +373,10 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
     a.o_acc = scratch + fck::kDecodeScratchTickets;
     a.lse_acc = a.o_acc + part_rows * dv;
     a.o = o;
-    g_kernel = uniform ? "splitkv_decode_kernel<uniform_page,fused>" : "splitkv_decode_kernel<row_lookup,fused>";
-    return launch_status(fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream)),
-                         "FmhaFwdSplitKV (fused) launch");
+    int hpw = 1;
+    const hipError_t e = fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream), &hpw);
+    name_decode_kernel(uniform, hpw, false, false, false, true);
+    return launch_status(e, "FmhaFwdSplitKV (fused) launch");
 }
 
 int fck_fmha_fused_reset(void* stream)
@@ -425,7 +448,35 @@ int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* kne
                           int64_t seqlen_k_cache, int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, int32_t dtype,
                           void* stream)
 {
+    return fck_fmha_fwd_appendkv_attrs(q, k_cache, v_cache, knew, vnew, seqlen_k, cu_seqlens_knew, seqlen_knew, rotary_cos, rotary_sin,
+                                       rotary_dim, rope_mode, has_mask, block_table, batch_stride_block_table, page_block_size,
+                                       cache_batch_idx, seqlen_k_cache, batch, hq, hk, d, dv, dtype, nullptr, stream);
+}
+
+int fck_fmha_fwd_appendkv_attrs(void* q, void* k_cache, void* v_cache, const void* knew, const void* vnew, const int32_t* seqlen_k,
+                                const int32_t* cu_seqlens_knew, int64_t seqlen_knew, const void* rotary_cos, const void* rotary_sin,
+                                int64_t rotary_dim, int32_t rope_mode, int32_t has_mask, const int32_t* block_table,
+                                int64_t batch_stride_block_table, int64_t page_block_size, const int32_t* cache_batch_idx,
+                                int64_t seqlen_k_cache, int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, int32_t dtype,
+                                const fck_fmha_attrs* attrs, void* stream)
+{
     g_err[0] = 0;
+    float k_descale = 1.f, v_descale = 1.f;
+    int32_t kv8 = 0;
+    if (attrs) {
+        if (attrs->size != sizeof(fck_fmha_attrs))
+            return fail(FCK_ERR_INVALID_ARGUMENT, "fck_fmha_attrs.size is %u, this library's struct has %zu bytes", attrs->size, sizeof(fck_fmha_attrs));
+        if (attrs->bias_type != 0 || attrs->bias || attrs->logits_soft_cap != 0.f)
+            return fail(FCK_ERR_INVALID_ARGUMENT, "appendKV takes no bias / soft cap: only kv_dtype, k_descale and v_descale of fck_fmha_attrs apply");
+        if (attrs->kv_dtype != 0) {
+            if (attrs->kv_dtype != FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: only 0 (same as knew) and FLOAT8 (1)", attrs->kv_dtype);
+            k_descale = attrs->k_descale == 0.f ? 1.f : attrs->k_descale;
+            v_descale = attrs->v_descale == 0.f ? 1.f : attrs->v_descale;
+            if (!(k_descale > 0.f) || !std::isfinite(k_descale) || !(v_descale > 0.f) || !std::isfinite(v_descale))
+                return fail(FCK_ERR_INVALID_ARGUMENT, "k_descale and v_descale must be positive and finite (0: 1)");
+            kv8 = 1;
+        }
+    }
     if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16)
         return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
     if (!k_cache || !v_cache || !knew || !vnew || !seqlen_k) return fail(FCK_ERR_INVALID_ARGUMENT, "k_cache, v_cache, knew, vnew and seqlen_k must not be null");
@@ -468,6 +519,10 @@ int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, const void* kne
     a.hk = (int32_t)hk;
     a.d = (int32_t)d;
     a.dv = (int32_t)dv;
+    a.kv8 = kv8;
+    a.k_descale = k_descale;
+    a.v_descale = v_descale;
+    if (kv8) return launch_status(fck::launch_appendkv_fp8(a, dtype, (int)seqlen_knew, static_cast<hipStream_t>(stream)), "FmhaFwdAppendKV (fp8 cache) launch");
     return launch_status(fck::launch_appendkv(a, dtype, (int)seqlen_knew, static_cast<hipStream_t>(stream)), "FmhaFwdAppendKV launch");
 }
 
@@ -489,6 +544,12 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t
         // head dims other than 64 / 128 / 256, or qk_head_dim != v_head_dim: the register-staged kernel pads them
         a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
         g_kernel = uniform ? "prefill_kernel<uniform_page,padded_head_dim>" : "prefill_kernel<row_lookup,padded_head_dim>";
+        return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+    }
+    if (a.kv8) {
+        // an fp8 cache is widened on its way into LDS, which only the register-staged kernel can do
+        a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
+        g_kernel = uniform ? "prefill_kernel<uniform_page,kv_fp8>" : "prefill_kernel<row_lookup,kv_fp8>";
         return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }
     if (a.mod.active()) {
@@ -547,7 +608,7 @@ int fck_fmha_fwd_attrs(const void* q, const void* k, const void* v, const void* 
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
-    if (int rc = no_kv_dtype(attrs)) return rc;
+    if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
     a.kv.page_shift = -1;
     a.kv.seqlen_k_ptr = seqlen_k_ptr;  // group mode: logical key counts of padded packed sequences
     if (seqstart_q) {
@@ -601,7 +662,7 @@ int fck_fmha_batch_prefill_attrs(const void* q, const void* k_cache, const void*
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
-    if (int rc = no_kv_dtype(attrs)) return rc;
+    if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
     a.kv.mode = 3;
     a.kv.kv_indptr = kv_indptr;
     a.kv.kv_page_indices = kv_page_indices;
@@ -654,7 +715,7 @@ int fck_fmha_fwd_pagedkv_attrs(const void* q, const void* k_cache, const void* v
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
-    if (int rc = no_kv_dtype(attrs)) return rc;
+    if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
     a.kv.mode = 2;
     a.kv.block_table = block_table;
     a.kv.block_table_stride = (int32_t)batch_stride_block_table;

@@ -78,6 +78,8 @@ struct AppendKvArgs {
     const int32_t* cache_batch_idx;
     int64_t seqlen_k_cache;
     int32_t batch, hq, hk, d, dv;
+    int32_t kv8;                 // the caches hold e4m3 bytes: cache = fp8(value / descale)
+    float k_descale, v_descale;
 };
 
 struct PrefillArgs {
@@ -94,6 +96,8 @@ struct PrefillArgs {
     int64_t window_left, window_right;
     ScoreMod mod;  // bias / ALiBi / soft cap; all zero: none (only the 4-wave kernel of prefill.hip applies them)
     int32_t d, dv;  // head dims of Q/K and of V/O as stored; other than the kernel's D only in the 4-wave kernel of prefill.hip
+    int32_t kv8;      // K and V are fp8 (e4m3); the K scale is folded into scale_log2 / mod.scale by the caller (4-wave kernel only)
+    float v_descale;  // factor on the output (1 unless V is quantised)
 };
 
 // arguments of the paged-cache checker: a block table (block_table != nullptr: seqlen_k, block_table_stride) or a page
@@ -112,8 +116,9 @@ struct ValidateArgs {
 hipError_t launch_validate_paged(const ValidateArgs& a, hipStream_t st);
 hipError_t launch_clear_tickets(uint32_t* tickets, int n, hipStream_t st);
 
+// heads_per_workgroup (may be null): receives the kernel variant the launcher took, 1 or 2 KV heads per workgroup
 hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page, int num_cu,
-                                 hipStream_t st);
+                                 hipStream_t st, int* heads_per_workgroup = nullptr);
 // Device memory the fused split-KV entry point uses instead of a caller-owned workspace: a fixed array in the library
 // (one copy per GPU): kDecodeScratchTickets arrival counters (self-resetting), then the partial results.
 constexpr int64_t kDecodeScratchTickets = 16384;
@@ -124,6 +129,8 @@ hipError_t decode_scratch(float** ptr);
 int splitkv_decode_m_tiles(int d, int rows_max);
 hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st);
 hipError_t launch_appendkv(const AppendKvArgs& a, int dtype, int max_new, hipStream_t st);
+// a.kv8: the caches hold e4m3 bytes
+hipError_t launch_appendkv_fp8(const AppendKvArgs& a, int dtype, int max_new, hipStream_t st);
 hipError_t launch_prefill(const PrefillArgs& a, int d, int dtype, bool uniform_page, hipStream_t st);
 // Tiles of a sequence whose first rows the direct-to-LDS prefill kernels cache in LDS; tiles past them are looked up one
 // by one.

@@ -13,6 +13,8 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
+#include <type_traits>
+
 namespace fck {
 
 template <int D>
@@ -36,9 +38,13 @@ constexpr size_t prefill_lds_bytes()
 // kPad: the stored head dims (a.d for Q/K, a.dv for V/O; multiples of 8) are smaller than D.  Rows are a.d / a.dv
 // elements apart and the 16-byte pieces past a row's end are zeros instead of loads: zero columns of Q and K add
 // nothing to a score, zero columns of V give output columns that are not stored.
-template <typename T, int D, bool kUniformPage, bool kMod = false, bool kPad = false>
+// kKv8: K and V are stored as fp8 (e4m3, one byte per element, static per-tensor scales) and widened to T on their way
+// into LDS; a lane then loads 8 bytes where the 16-bit path loads 16.  The K scale arrives folded into the softmax
+// scale, the V scale multiplies the output.  Always together with kMod (the identity when no modifier is set).
+template <typename T, int D, bool kUniformPage, bool kMod = false, bool kPad = false, bool kKv8 = false>
 __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const PrefillArgs a)
 {
+    static_assert(!kKv8 || (kMod && !kPad), "fp8 cache: the general kernel, stored head dims equal to D");
     const int dq = kPad ? a.d : D;    // elements per stored Q / K row
     const int dvs = kPad ? a.dv : D;  // elements per stored V / O row
     typedef PrefillShape<D> S;
@@ -114,15 +120,27 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
         for (int j = 0; j < 16; ++j) oacc[i][j] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
-    const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k);
-    const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v);
+    typedef typename std::conditional<kKv8, uint8_t, uint16_t>::type kv_elem;
+    const kv_elem* kp = reinterpret_cast<const kv_elem*>(a.k);
+    const kv_elem* vp = reinterpret_cast<const kv_elem*>(a.v);
     const int last_key = sk_b - 1;
     // this thread's piece u of a K / V row: offset inside the row's cache line-up, or zeros when the row ends before it
-    auto load_piece = [&](const uint16_t* base, int64_t row, int c, int dim) -> u32x4_t {
+    auto load_piece = [&](const kv_elem* base, int64_t row, int c, int dim) -> u32x4_t {
         if constexpr (kPad) {
             if (c * 8 >= dim) return u32x4_t{0u, 0u, 0u, 0u};
         }
-        return ldg16(base + (row * a.hk + hkv) * dim + c * 8);
+        if constexpr (kKv8) {
+            const u32x2_t v = *reinterpret_cast<const u32x2_t*>(base + (row * a.hk + hkv) * dim + c * 8);
+            return u32x4_t{v[0], v[1], 0u, 0u};
+        } else {
+            return ldg16(base + (row * a.hk + hkv) * dim + c * 8);
+        }
+    };
+    auto staged = [](u32x4_t v) -> u32x4_t {
+        if constexpr (kKv8)
+            return fp8x8_to_t<T>(v);
+        else
+            return v;
     };
 
     // global -> LDS copy assignment: 16-byte chunk (row, c) per thread and step
@@ -164,8 +182,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
         char FCK_LDS* vd = lds + (2 + buf) * S::TILEB;
 #pragma unroll
         for (int u = 0; u < S::LD; ++u) {
-            *(u32x4_t FCK_LDS*)(kd + cp_koff[u]) = kreg[u];
-            *(u32x4_t FCK_LDS*)(vd + cp_voff[u]) = vreg[u];
+            *(u32x4_t FCK_LDS*)(kd + cp_koff[u]) = staged(kreg[u]);
+            *(u32x4_t FCK_LDS*)(vd + cp_voff[u]) = staged(vreg[u]);
         }
     };
 
@@ -289,7 +307,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
     // ---- epilogue ----------------------------------------------------------------------------------------------------
     l_run = pair32_sum(l_run);
     if (row_ok) {
-        const float inv = (l_run == 0.f) ? 0.f : 1.f / l_run;
+        float inv = (l_run == 0.f) ? 0.f : 1.f / l_run;
+        if constexpr (kKv8) inv *= a.v_descale;
         uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * dvs;
 #pragma unroll
         for (int dvb = 0; dvb < S::DVB; ++dvb)
@@ -311,6 +330,11 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
 {
     const dim3 grid(a.m_tiles, a.hq, a.batch);
     constexpr size_t lds = prefill_lds_bytes<D>();
+    if (a.kv8) {  // fp8 cache: the general kernel with the widening load (the caller refuses padded head dims)
+        if (a.d != D || a.dv != D) return hipErrorInvalidValue;
+        if (uniform) return launch_with_lds<prefill_kernel<T, D, true, true, false, true>>(grid, dim3(256), lds, st, a);
+        return launch_with_lds<prefill_kernel<T, D, false, true, false, true>>(grid, dim3(256), lds, st, a);
+    }
     if (a.d != D || a.dv != D) {  // padded head dims: the general kernel (modifiers on, identity when there are none)
         if (uniform) return launch_with_lds<prefill_kernel<T, D, true, true, true>>(grid, dim3(256), lds, st, a);
         return launch_with_lds<prefill_kernel<T, D, false, true, true>>(grid, dim3(256), lds, st, a);

@@ -617,8 +617,9 @@ static bool use_head_pairs(const SplitKvArgs& a, int m_tiles, int num_cu)
 }
 
 template <typename T, int D>
-static hipError_t launch_mb(SplitKvArgs a, int rows_max, bool uniform, int num_cu, hipStream_t st)
+static hipError_t launch_mb(SplitKvArgs a, int rows_max, bool uniform, int num_cu, hipStream_t st, int* heads_per_workgroup)
 {
+    *heads_per_workgroup = 1;
     // 8 waves (2 per SIMD, 256 VGPRs each) when one 16-row block is enough; 4 waves (512 VGPRs) when a lane carries
     // the accumulators of several row blocks or of a 256-wide head.
     a.m_tiles = splitkv_decode_m_tiles(D, rows_max);
@@ -638,6 +639,7 @@ static hipError_t launch_mb(SplitKvArgs a, int rows_max, bool uniform, int num_c
         if (rows_max <= 16) {
             if (use_head_pairs(a, 1, num_cu)) {
                 set_order(2);
+                *heads_per_workgroup = 2;
                 return launch_cfg<T, D, 8, 1, 2>(a, uniform, st);
             }
             return launch_cfg<T, D, 8, 1, 1>(a, uniform, st);
@@ -648,12 +650,12 @@ static hipError_t launch_mb(SplitKvArgs a, int rows_max, bool uniform, int num_c
 }
 
 template <typename T>
-static hipError_t launch_d(const SplitKvArgs& a, int d, int rows_max, bool uniform, int num_cu, hipStream_t st)
+static hipError_t launch_d(const SplitKvArgs& a, int d, int rows_max, bool uniform, int num_cu, hipStream_t st, int* hpw)
 {
     switch (d) {
-    case 64: return launch_mb<T, 64>(a, rows_max, uniform, num_cu, st);
-    case 128: return launch_mb<T, 128>(a, rows_max, uniform, num_cu, st);
-    case 256: return launch_mb<T, 256>(a, rows_max, uniform, num_cu, st);
+    case 64: return launch_mb<T, 64>(a, rows_max, uniform, num_cu, st, hpw);
+    case 128: return launch_mb<T, 128>(a, rows_max, uniform, num_cu, st, hpw);
+    case 256: return launch_mb<T, 256>(a, rows_max, uniform, num_cu, st, hpw);
     }
     return hipErrorInvalidValue;
 }
@@ -665,10 +667,13 @@ int splitkv_decode_m_tiles(int d, int rows_max)
 }
 
 hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page, int num_cu,
-                                 hipStream_t st)
+                                 hipStream_t st, int* heads_per_workgroup)
 {
-    if (dtype == 4) return launch_d<BF16>(a, d, rows_max, uniform_page, num_cu, st);
-    return launch_d<FP16>(a, d, rows_max, uniform_page, num_cu, st);
+    int hpw = 1;
+    const hipError_t e = dtype == 4 ? launch_d<BF16>(a, d, rows_max, uniform_page, num_cu, st, &hpw)
+                                    : launch_d<FP16>(a, d, rows_max, uniform_page, num_cu, st, &hpw);
+    if (heads_per_workgroup) *heads_per_workgroup = hpw;
+    return e;
 }
 
 }  // namespace fck

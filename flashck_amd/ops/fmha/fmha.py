@@ -163,6 +163,7 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
         if bias.shape[-2] != rows or bias.shape[-1] < min_cols:
             raise ValueError(f"bias {tuple(bias.shape)} must have {rows} rows and at least {min_cols} columns")
         a.bias_type = 1
+        a.bias_cols = bias.shape[-1]
         a.bias = bias.data_ptr()
         a.bias_row_stride = bias.stride(-2)
         a.bias_head_stride = bias.stride(-3) if bias.shape[-3] > 1 else 0
@@ -460,18 +461,20 @@ def fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype, cu_seqlens_q=None, max_seqle
 
 def fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, *, cu_seqlens_knew=None, max_seqlen_knew: int = 0,
                       rotary_cos=None, rotary_sin=None, rope_mode: int = ROPE_NONE, has_mask: bool = True,
-                      block_table=None, cache_batch_idx=None) -> None:
+                      block_table=None, cache_batch_idx=None, k_descale: float = 1.0, v_descale: float = 1.0) -> None:
     """Rotate knew (and q, in place) and append knew/vnew to the cache behind seqlen_k[b] tokens; in place.
 
     knew/vnew/q are packed [total_new, H, D] with cu_seqlens_knew, or [B, n, H, D] with n new tokens everywhere.
     seqlen_k is NOT advanced: the caller adds the new counts, as with the ck_tile kernel.
+    torch.float8_e4m3fn caches are written quantised with the static scales: cache = fp8(x / descale), saturating.
     """
     packed = cu_seqlens_knew is not None
     _check_tensor("knew", knew, ndim=3 if packed else 4)
     _check_tensor("vnew", vnew, dtype=knew.dtype, ndim=3 if packed else 4)
     _check_tensor("q", q, dtype=knew.dtype, ndim=3 if packed else 4, optional=True)
-    _check_tensor("k_cache", k_cache, dtype=knew.dtype, ndim=4)
-    _check_tensor("v_cache", v_cache, dtype=knew.dtype, ndim=4)
+    kv_fp8 = isinstance(k_cache, torch.Tensor) and k_cache.dtype == torch.float8_e4m3fn
+    _check_tensor("k_cache", k_cache, dtype=torch.float8_e4m3fn if kv_fp8 else knew.dtype, ndim=4)
+    _check_tensor("v_cache", v_cache, dtype=torch.float8_e4m3fn if kv_fp8 else knew.dtype, ndim=4)
     _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1)
     for name, t in (("cu_seqlens_knew", cu_seqlens_knew), ("block_table", block_table), ("cache_batch_idx", cache_batch_idx)):
         _check_tensor(name, t, dtype=torch.int32, optional=True)
@@ -515,19 +518,31 @@ def fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, *, cu_seqlens_k
                            page_size=page, check=True)
     else:
         stride, page, rows = 0, 0, k_cache.shape[1]
-    _call("fck_fmha_fwd_appendkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(knew), _ptr(vnew), _ptr(seqlen_k),
-          _ptr(cu_seqlens_knew), n, _ptr(rotary_cos), _ptr(rotary_sin), rotary_dim, rope_mode, int(bool(has_mask)),
-          _ptr(block_table), stride, page, _ptr(cache_batch_idx), rows, B, Hq, Hk, D, Dv, _dtype_id(knew), _stream())
+    args = (_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(knew), _ptr(vnew), _ptr(seqlen_k), _ptr(cu_seqlens_knew), n,
+            _ptr(rotary_cos), _ptr(rotary_sin), rotary_dim, rope_mode, int(bool(has_mask)), _ptr(block_table), stride, page,
+            _ptr(cache_batch_idx), rows, B, Hq, Hk, D, Dv, _dtype_id(knew))
+    if kv_fp8:
+        if not (float(k_descale) > 0.0 and float(v_descale) > 0.0 and math.isfinite(k_descale) and math.isfinite(v_descale)):
+            raise ValueError("k_descale and v_descale must be positive and finite")
+        at = _lib.Attrs()
+        at.size = ctypes.sizeof(_lib.Attrs)
+        at.kv_dtype, at.k_descale, at.v_descale = 1, float(k_descale), float(v_descale)  # flashck::DataType FLOAT8
+        _call("fck_fmha_fwd_appendkv_attrs", *args, ctypes.byref(at), _stream())
+    else:
+        _call("fck_fmha_fwd_appendkv", *args, _stream())
 
 
 def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_indices, kv_last_page_lens=None, *,
                        max_seqlen_q: int, scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0),
-                       out=None, bias=None, alibi_slopes=None, logits_soft_cap: float = 0.0) -> torch.Tensor:
+                       out=None, bias=None, alibi_slopes=None, logits_soft_cap: float = 0.0, k_descale: float = 1.0,
+                       v_descale: float = 1.0) -> torch.Tensor:
     """Varlen prefill over a page list: q [total_q,Hq,D]; sequence b owns pages
-    kv_page_indices[kv_indptr[b]:kv_indptr[b+1]] of the cache [num_pages, page_size, Hk, D]."""
+    kv_page_indices[kv_indptr[b]:kv_indptr[b+1]] of the cache [num_pages, page_size, Hk, D].  The caches may be
+    torch.float8_e4m3fn with the static scales k_descale / v_descale (value = descale * stored)."""
     _check_tensor("q", q, ndim=3)
-    _check_tensor("k_cache", k_cache, dtype=q.dtype, ndim=4)
-    _check_tensor("v_cache", v_cache, dtype=q.dtype, ndim=4)
+    kv_fp8 = isinstance(k_cache, torch.Tensor) and k_cache.dtype == torch.float8_e4m3fn
+    _check_tensor("k_cache", k_cache, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype, ndim=4)
+    _check_tensor("v_cache", v_cache, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype, ndim=4)
     for name, t in (("cu_seqlens_q", cu_seqlens_q), ("kv_indptr", kv_indptr), ("kv_page_indices", kv_page_indices)):
         _check_tensor(name, t, dtype=torch.int32, ndim=1)
     _check_tensor("kv_last_page_lens", kv_last_page_lens, dtype=torch.int32, ndim=1, optional=True)
@@ -543,7 +558,7 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
     wl, wr = _window(window)
     _debug_validate(kv_indptr=kv_indptr, kv_page_indices=kv_page_indices, kv_last_page_lens=kv_last_page_lens,
                     num_total_pages=num_pages, page_size=page)
-    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1)
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1, kv_fp8, k_descale, v_descale)
     if at is None:
         _call("fck_fmha_batch_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
               _ptr(kv_page_indices), _ptr(kv_last_page_lens), num_pages, page, B, Hq, Hk, D, Dv, max_seqlen_q,
@@ -558,12 +573,14 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
 
 def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q=None, max_seqlen_q: int = 0,
                      scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0), out=None, bias=None,
-                     alibi_slopes=None, logits_soft_cap: float = 0.0) -> torch.Tensor:
-    """Prefill over a block table (no splits): q [B,sq,Hq,D] or packed [total_q,Hq,D]."""
+                     alibi_slopes=None, logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0) -> torch.Tensor:
+    """Prefill over a block table (no splits): q [B,sq,Hq,D] or packed [total_q,Hq,D].  The caches may be
+    torch.float8_e4m3fn with the static scales k_descale / v_descale (value = descale * stored)."""
     group = cu_seqlens_q is not None
     _check_tensor("q", q, ndim=3 if group else 4)
-    _check_tensor("k_cache", k_cache, dtype=q.dtype, ndim=4)
-    _check_tensor("v_cache", v_cache, dtype=q.dtype, ndim=4)
+    kv_fp8 = isinstance(k_cache, torch.Tensor) and k_cache.dtype == torch.float8_e4m3fn
+    _check_tensor("k_cache", k_cache, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype, ndim=4)
+    _check_tensor("v_cache", v_cache, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype, ndim=4)
     _check_tensor("seqlen_k", seqlen_k, dtype=torch.int32, ndim=1)
     _check_tensor("block_table", block_table, dtype=torch.int32, ndim=2)
     _check_tensor("cu_seqlens_q", cu_seqlens_q, dtype=torch.int32, ndim=1, optional=True)
@@ -581,7 +598,7 @@ def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q
     o = _out("out", out, (*q.shape[:-1], Dv), q.dtype, q)
     wl, wr = _window(window)
     _debug_validate(seqlen_k=seqlen_k, block_table=block_table, num_total_pages=k_cache.shape[0], page_size=page)
-    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, q.shape[0] if group else sq, 1)
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, q.shape[0] if group else sq, 1, kv_fp8, k_descale, v_descale)
     if at is None:
         _call("fck_fmha_fwd_pagedkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
               _ptr(block_table), block_table.shape[1], page, B, sq, Hq, Hk, D, Dv, max_seqlen_q or sq, _scale(scale, D), wl, wr,
@@ -728,7 +745,7 @@ class DecodeWorkspace:
 def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_knew=None,
                      max_seqlen_knew: int = 0, rotary_cos=None, rotary_sin=None, rope_mode: int = ROPE_NONE,
                      num_splits: int = 0, max_seqlen_k: int = 0, scale: float = 0.0, window_left: int = -1,
-                     workspace: Optional[DecodeWorkspace] = None, out=None):
+                     workspace: Optional[DecodeWorkspace] = None, out=None, k_descale: float = 1.0, v_descale: float = 1.0):
     """One serving step over a paged cache: append the new tokens, then attend from them.
 
     The caller side of the split-KV path, FmhaKind::FwdAppendKV -> FwdSplitKV -> FwdSplitKVCombine
@@ -741,6 +758,8 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
          its own position (bottom-right causal; window_left >= 0 adds a sliding window) - and the LSE combine.
     q/knew/vnew are [B, n, H, D] (n new tokens everywhere) or packed [total_new, H, D] with cu_seqlens_knew and
     max_seqlen_knew.  Nothing is read back from the GPU, so a step only enqueues work on the current stream.
+    With torch.float8_e4m3fn caches the new rows are quantised on their way in and dequantised by the attention
+    kernel, both with the static scales k_descale / v_descale.
 
     Returns (o, seqlen_k_new): o has q's shape (with Dv); seqlen_k_new = seqlen_k + n_b lives in the workspace and is
     overwritten by the next step; seqlen_k itself is not modified.
@@ -761,7 +780,8 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
         n = q.shape[1]
     fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, cu_seqlens_knew=cu_seqlens_knew, max_seqlen_knew=n,
                       rotary_cos=rotary_cos, rotary_sin=rotary_sin, rope_mode=rope_mode, has_mask=True,
-                      block_table=block_table)
+                      block_table=block_table, k_descale=k_descale, v_descale=v_descale)
+    kv_fp8 = k_cache.dtype == torch.float8_e4m3fn
     seqlen_new, counts = ws.lengths(B, seqlen_k.device)
     if packed:
         torch.sub(cu_seqlens_knew[1:], cu_seqlens_knew[:-1], out=counts)
@@ -772,7 +792,7 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * page  # what the block table can address
         num_splits, decode_variant = _auto_num_splits(B, Hq, Hk, n, max_seqlen_k, D, page, q.dtype)
-        decode_variant = _usable_variant(decode_variant, Hq, Hk, n, D, Dv)
+        decode_variant = _usable_variant(decode_variant, Hq, Hk, n, D, Dv, plain=not kv_fp8)
     else:
         decode_variant = 0
     # a lone new token sees every key: no mask needed unless a sliding window is asked for
@@ -784,7 +804,8 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
     o_acc, lse_acc = ws.partials(shape_batch, Hq, num_splits, shape_sq, Dv, q.device)
     fmha_fwd_splitkv(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_new, block_table=block_table,
                      cu_seqlens_q=cu_seqlens_knew, max_seqlen_q=n if packed else 0, scale=scale, mask_type=mask_type,
-                     window=window, o_acc=o_acc, lse_acc=lse_acc, decode_variant=decode_variant)
+                     window=window, o_acc=o_acc, lse_acc=lse_acc, decode_variant=decode_variant, k_descale=k_descale,
+                     v_descale=v_descale)
     o = fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_knew, max_seqlen_q=n if packed else 0,
                                  out=out)
     return o, seqlen_new

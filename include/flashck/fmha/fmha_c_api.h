@@ -95,6 +95,13 @@ typedef struct fck_fmha_attrs {
      * 2 = two adjacent KV heads per workgroup (16-key tiles, 512-byte row pieces; needs an even kv_num_heads, at most
      * 16 packed query rows, head dim <= 128 and no bias / soft cap).  A variant the problem cannot take is an error. */
     int32_t decode_variant;
+    /* Prefill kernel variant, likewise: 0 = the library chooses; see fck_fmha_fwd for the values.  A variant the problem
+     * cannot take is an error. */
+    int32_t prefill_variant;
+    /* ELEMENTWISE_BIAS: columns a bias row holds.  A key index is clamped to the last of them before the bias is read,
+     * so a bias narrower than a sequence's key count is never read out of bounds (the scores of such keys then use
+     * the last column).  0: not stated, only the sequence's own key count bounds the reads. */
+    int64_t bias_cols;
 } fck_fmha_attrs;
 
 #define FCK_OK 0
@@ -250,6 +257,20 @@ FCK_EXPORT int fck_fmha_fwd_appendkv(void* q, void* k_cache, void* v_cache, cons
                                      const int32_t* cache_batch_idx, int64_t seqlen_k_cache, int64_t batch,
                                      int64_t q_num_heads, int64_t kv_num_heads, int64_t qk_head_dim,
                                      int64_t v_head_dim, int32_t dtype, void* stream);
+
+/* The same for a quantised cache: attrs->kv_dtype = FCK_DTYPE_FP8 makes k_cache / v_cache one e4m3 byte per element,
+ * written as fp8(x / k_descale) resp. fp8(x / v_descale) with round-to-nearest-even and saturation at +-448, where x is
+ * the element a cache of `dtype` would receive (the rotated K row rounded to `dtype`, the V row as given): the static
+ * quantisation of the reference's fp8 type configuration (core/module/kernels/attention_kernels/fmha_common_jinja.h:157-171,
+ * is_static_quant).  knew, vnew and q keep `dtype`.  The bias / soft cap fields of `attrs` must be unset. */
+FCK_EXPORT int fck_fmha_fwd_appendkv_attrs(void* q, void* k_cache, void* v_cache, const void* knew, const void* vnew,
+                                           const int32_t* seqlen_k, const int32_t* cu_seqlens_knew, int64_t seqlen_knew,
+                                           const void* rotary_cos, const void* rotary_sin, int64_t rotary_dim,
+                                           int32_t rope_mode, int32_t has_mask, const int32_t* block_table,
+                                           int64_t batch_stride_block_table, int64_t page_block_size,
+                                           const int32_t* cache_batch_idx, int64_t seqlen_k_cache, int64_t batch,
+                                           int64_t q_num_heads, int64_t kv_num_heads, int64_t qk_head_dim,
+                                           int64_t v_head_dim, int32_t dtype, const fck_fmha_attrs* attrs, void* stream);
 
 /*
  * Varlen batch prefill over a page list.  FlashCK's problem definition:

@@ -112,6 +112,37 @@ float fck_orc_fp8_to_f32(uint8_t x)
     return (x & 0x80) ? -v : v;
 }
 
+/* fp32 -> OCP e4m3, round to nearest even, saturating: finite values beyond +-448 give +-448 (0x7e), NaN and infinities
+   give NaN (0x7f).  The software conversion of ck_tile (ck_tile/core/numeric/float8.hpp:249-470, run_cast_to_f8 with
+   clip = true, no stochastic rounding) and, on the device, fmed3(x, 448, -448) on finite values followed by the RNE
+   conversion instruction (same file :600-662). */
+uint8_t fck_orc_f32_to_fp8(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    if ((u & 0x7f800000u) == 0x7f800000u) return (uint8_t)(sign | 0x7fu);
+    float a = fabsf(f);
+    if (a >= 448.f) return (uint8_t)(sign | 0x7eu);
+    if (a == 0.f) return sign;
+    /* the grid of representable values around a: spacing 2^(e-3) for a in [2^e, 2^(e+1)), e >= -6; 2^-9 below 2^-6 */
+    int e;
+    (void)frexpf(a, &e); /* a = m * 2^e, m in [0.5, 1) -> a in [2^(e-1), 2^e) */
+    int ex = e - 1;
+    if (ex < -6) ex = -6;
+    const float q = ldexpf(a, 3 - ex);       /* a in units of the spacing: exact (a power-of-two scaling) */
+    float r = rintf(q);                      /* round to nearest even (default rounding mode) */
+    /* r in [0, 16]; r == 16 means the value rounded up into the next binade */
+    int mant = (int)r, be = ex + 7;          /* biased exponent for normal numbers */
+    if (ex == -6 && mant < 8) return (uint8_t)(sign | (uint8_t)mant); /* subnormal (or zero) */
+    if (mant == 16) {
+        mant = 8;
+        be += 1;
+    }
+    if (be > 15 || (be == 15 && mant - 8 > 6)) return (uint8_t)(sign | 0x7eu); /* cannot happen below 448; kept for safety */
+    return (uint8_t)(sign | (uint8_t)(be << 3) | (uint8_t)(mant - 8));
+}
+
 static inline float ld(const void* base, int64_t idx, int dtype)
 {
     uint16_t x = ((const uint16_t*)base)[idx];
@@ -520,9 +551,11 @@ int fck_orc_appendkv(void* q, void* k_cache, void* v_cache, const void* knew, co
                      const int32_t* cu_seqlens_knew, const void* cos_tab, const void* sin_tab, int rotary_dim,
                      int rope_mode, int has_mask, const int32_t* block_table, int block_table_stride, int page_size,
                      const int32_t* cache_batch_idx, int64_t cache_batch_stride_rows, int batch, int hq, int hk, int d,
-                     int dv, int dtype)
+                     int dv, int dtype, int kv_dtype, float k_descale, float v_descale)
 {
     if (dtype != FCK_ORC_BF16 && dtype != FCK_ORC_FP16) return -1;
+    if (kv_dtype != 0 && kv_dtype != FCK_ORC_FP8) return -1;
+    const int kv8 = kv_dtype == FCK_ORC_FP8;
     uint16_t* tmp = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)d);
     for (int b = 0; b < batch; ++b) {
         const int n0 = cu_seqlens_knew[b], n = cu_seqlens_knew[b + 1] - n0;
@@ -539,6 +572,19 @@ int fck_orc_appendkv(void* q, void* k_cache, void* v_cache, const void* knew, co
             }
             for (int h = 0; h < hk; ++h) {
                 const uint16_t* src = (const uint16_t*)knew + ((int64_t)(n0 + i) * hk + h) * d;
+                if (kv8) {
+                    /* quantised cache: the row a 16-bit cache would hold (rotated, rounded to T), divided by the static
+                       scale and converted to e4m3; V likewise without the rotation */
+                    if (rope_mode != FCK_ORC_ROPE_NONE)
+                        rope_row(src, tmp, d, cos_tab, sin_tab, t, rotary_dim, rope_mode, dtype);
+                    else
+                        memcpy(tmp, src, sizeof(uint16_t) * (size_t)d);
+                    uint8_t* kd = (uint8_t*)k_cache + (prow * hk + h) * d;
+                    for (int c = 0; c < d; ++c) kd[c] = fck_orc_f32_to_fp8(ld(tmp, c, dtype) / k_descale);
+                    uint8_t* vd = (uint8_t*)v_cache + (prow * hk + h) * dv;
+                    for (int c = 0; c < dv; ++c) vd[c] = fck_orc_f32_to_fp8(ld(vnew, ((int64_t)(n0 + i) * hk + h) * dv + c, dtype) / v_descale);
+                    continue;
+                }
                 uint16_t* dst = (uint16_t*)k_cache + (prow * hk + h) * d;
                 if (rope_mode != FCK_ORC_ROPE_NONE) {
                     rope_row(src, tmp, d, cos_tab, sin_tab, t, rotary_dim, rope_mode, dtype);

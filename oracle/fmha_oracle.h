@@ -104,7 +104,11 @@ int fck_orc_appendkv(void* q, void* k_cache, void* v_cache, const void* knew, co
                      const void* sin_tab, int rotary_dim, int rope_mode, int has_mask,
                      const int32_t* block_table, int block_table_stride, int page_size,
                      const int32_t* cache_batch_idx, int64_t cache_batch_stride_rows, int batch, int hq,
-                     int hk, int d, int dv, int dtype);
+                     int hk, int d, int dv, int dtype, int kv_dtype, float k_descale, float v_descale);
+/* kv_dtype FCK_ORC_FP8: the caches hold one e4m3 byte per element: cache = fp8(value a 16-bit cache would hold / descale) */
+
+/* fp32 -> e4m3 byte: round to nearest even, finite overflow saturates to +-448, NaN / inf give NaN */
+uint8_t fck_orc_f32_to_fp8(float f);
 
 /* Gather one sequence's first n rows of a paged cache into dst [n, Hk, D]. */
 int fck_orc_gather_paged(const void* cache, const int32_t* pages, int page_size, int n, int hk, int d,

@@ -70,7 +70,10 @@ def lib():
         _lib.fck_orc_rope.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                       ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _lib.fck_orc_appendkv.argtypes = ([ctypes.c_void_p] * 9 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int,
-                                          ctypes.c_int, ctypes.c_void_p, ctypes.c_int64] + [ctypes.c_int] * 6)
+                                          ctypes.c_int, ctypes.c_void_p, ctypes.c_int64] + [ctypes.c_int] * 7
+                                         + [ctypes.c_float] * 2)
+        _lib.fck_orc_f32_to_fp8.restype = ctypes.c_uint8
+        _lib.fck_orc_f32_to_fp8.argtypes = [ctypes.c_float]
         _lib.fck_orc_gather_paged.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 5 + [ctypes.c_void_p]
     return _lib
 
@@ -227,9 +230,15 @@ def rope(x, pos, cos, sin, rope_mode=ROPE_HALF_ROTATED):
     return out
 
 
+def f32_to_fp8(x: float) -> int:
+    return lib().fck_orc_f32_to_fp8(x)
+
+
 def appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, cu_seqlens_knew, cos=None, sin=None,
-             rope_mode=ROPE_NONE, has_mask=True, block_table=None, cache_batch_idx=None):
-    """In place on q, k_cache, v_cache (CPU tensors)."""
+             rope_mode=ROPE_NONE, has_mask=True, block_table=None, cache_batch_idx=None, k_descale=1.0, v_descale=1.0):
+    """In place on q, k_cache, v_cache (CPU tensors).  torch.float8_e4m3fn caches are written quantised with the static
+    scales k_descale / v_descale."""
+    kv_dtype = FP8 if k_cache.dtype == torch.float8_e4m3fn else 0
     batch = seqlen_k.numel()
     hk, d = knew.shape[-2], knew.shape[-1]
     dv = vnew.shape[-1]
@@ -242,7 +251,7 @@ def appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, cu_seqlens_knew, cos=Non
     rc = lib().fck_orc_appendkv(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(knew), _ptr(vnew), _i32(seqlen_k),
                                 _i32(cu_seqlens_knew), _ptr(cos), _ptr(sin), rotary_dim, rope_mode, int(has_mask),
                                 _i32(block_table), stride, page, _i32(cache_batch_idx), cbs, batch, hq, hk, d, dv,
-                                dtype_id(knew.dtype))
+                                dtype_id(knew.dtype), kv_dtype, float(k_descale), float(v_descale))
     assert rc == 0, rc
 
 

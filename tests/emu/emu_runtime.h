@@ -225,6 +225,31 @@ inline float e4m3_to_f32(uint8_t b)
         v = ldexpf((float)(8 + m), e - 10);
     return s ? -v : v;
 }
+// fp32 -> e4m3, round to nearest even by search over the 127 positive finite codes (ties go to the even code, which
+// for adjacent codes is the even mantissa); beyond the largest finite value and for NaN / inf: NaN
+inline uint8_t f32_to_e4m3(float f)
+{
+    const uint8_t sign = std::signbit(f) ? 0x80 : 0;
+    const float a = fabsf(f);
+    if (!(a == a) || std::isinf(a)) return sign | 0x7f;
+    if (a >= 464.f) return sign | 0x7f;  // rounds past 448: not representable without saturation
+    int best = 0;
+    float best_err = a;  // code 0 = zero
+    for (int c = 1; c <= 0x7e; ++c) {
+        const float err = fabsf(e4m3_to_f32((uint8_t)c) - a);
+        if (err < best_err || (err == best_err && (c & 1) == 0)) {
+            best = c;
+            best_err = err;
+        }
+    }
+    return sign | (uint8_t)best;
+}
+inline int cvt_pk_fp8_f32(float a, float b, int old, bool hi)
+{
+    const uint32_t two = (uint32_t)f32_to_e4m3(a) | ((uint32_t)f32_to_e4m3(b) << 8);
+    const uint32_t o = (uint32_t)old;
+    return (int)(hi ? ((o & 0xffffu) | (two << 16)) : ((o & 0xffff0000u) | two));
+}
 inline emu_f32x2 cvt_pk_f32_fp8(int v, bool hi)
 {
     const uint32_t u = (uint32_t)v >> (hi ? 16 : 0);
@@ -245,5 +270,6 @@ inline emu_f32x2 cvt_pk_f32_fp8(int v, bool hi)
 #define __builtin_amdgcn_logf(x) log2f(x)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define __builtin_amdgcn_cvt_pk_f32_fp8(v, hi) emu::cvt_pk_f32_fp8((v), (hi))
+#define __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, hi) emu::cvt_pk_fp8_f32((a), (b), (old), (hi))
 #define __HIP_MEMORY_SCOPE_AGENT 0
 #define __hip_atomic_fetch_add(p, v, order, scope) __atomic_fetch_add((p), (v), __ATOMIC_SEQ_CST)

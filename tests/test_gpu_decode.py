@@ -75,7 +75,7 @@ def test_paged_decode_head_pairs(fmha, orc, dtype, d, page):
     kv["scale"] = 1 / math.sqrt(d)
     _run_paged(fmha, orc, kv, 4)
     from flashck_amd import _lib
-    assert b"splitkv_decode_kernel" in _lib.load().fck_fmha_last_kernel()
+    assert b"head_pairs" in _lib.load().fck_fmha_last_kernel()   # the name says which variant the launcher took
     _run_paged(fmha, orc, kv, 4, mask_type=2, window=(40, 0))  # sliding window: leading tiles are skipped
 
 

@@ -240,7 +240,12 @@ def test_fp8_cache_is_refused_where_no_kernel_reads_it(fmha):
     lib = _lib.load()
     at = _lib.Attrs()
     at.size, at.kv_dtype = ctypes.sizeof(_lib.Attrs), 1
-    x = torch.zeros(1, 4, 4, 64, dtype=torch.float16, device=helpers.DEVICE)
-    rc = lib.fck_fmha_fwd_attrs(x.data_ptr(), x.data_ptr(), x.data_ptr(), None, x.data_ptr(), None, None, None, 1, 4, 4, 4, 4, 64, 64,
+    x = torch.zeros(1, 4, 4, 128, dtype=torch.float16, device=helpers.DEVICE)
+    # head dims the kernels pad (qk 64, v 128) do not combine with an fp8 cache
+    rc = lib.fck_fmha_fwd_attrs(x.data_ptr(), x.data_ptr(), x.data_ptr(), None, x.data_ptr(), None, None, None, 1, 4, 4, 4, 4, 64, 128,
                                 4, 0.125, -1, -1, 0, 3, ctypes.byref(at), None)
-    assert rc == -2 and b"split-KV entry point only" in lib.fck_last_error()
+    assert rc == -2 and b"fp8 K/V cache needs" in lib.fck_last_error()
+    at.kv_dtype = 2   # only e4m3 (FLOAT8 = 1) is a cache type
+    rc = lib.fck_fmha_fwd_attrs(x.data_ptr(), x.data_ptr(), x.data_ptr(), None, x.data_ptr(), None, None, None, 1, 4, 4, 4, 4, 128, 128,
+                                4, 0.125, -1, -1, 0, 3, ctypes.byref(at), None)
+    assert rc == -2 and b"kv_dtype 2" in lib.fck_last_error()
