@@ -333,6 +333,41 @@ struct RowMod {
     }
 };
 
+// The modifiers that are pure arithmetic on a score (ALiBi, soft cap): RowMod without the elementwise bias, for the
+// kernels whose vector phase has no room for a load per score.  Same formulas, same results.
+struct ArithMod {
+    float slope;
+    int32_t zero, mode;
+    float scale, cap, cap_rcp;
+    bool alibi;
+
+    __device__ __forceinline__ void init(const ScoreMod& m, int b, int h, int i, int sq, int sk, uint32_t mask_type, int64_t wl, int64_t wr)
+    {
+        scale = m.scale;
+        cap = m.soft_cap;
+        cap_rcp = m.soft_cap > 0.f ? 1.f / m.soft_cap : 0.f;
+        alibi = m.bias_type == 2;
+        slope = 0.f;
+        zero = 0;
+        mode = alibi_mode(mask_type, wl, wr);
+        if (alibi) {
+            const float sl = reinterpret_cast<const float*>(m.bias)[(int64_t)b * m.batch_stride + h];
+            slope = mode == kAlibiVertical ? sl : -sl;
+            zero = mode == kAlibiBottomRight ? i + sk - sq : i;
+        }
+    }
+    __device__ __forceinline__ float score(float qk, int key) const
+    {
+        float x = qk * scale;
+        if (cap > 0.f) x = cap * fast_tanh(x * cap_rcp);
+        if (alibi) {
+            const int dist = mode == kAlibiVertical ? key : abs(zero - key);
+            x = __builtin_fmaf(slope, (float)dist, x);
+        }
+        return x * kLog2e;
+    }
+};
+
 // Where the K/V rows of one sequence live.  `table` == nullptr: rows are contiguous from base_row.
 // Otherwise logical key j sits at row table[j / page] * page + j % page.
 struct KvSeq {

@@ -552,21 +552,28 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t
         g_kernel = uniform ? "prefill_kernel<uniform_page,kv_fp8>" : "prefill_kernel<row_lookup,kv_fp8>";
         return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }
-    if (a.mod.active()) {
-        // bias, ALiBi and the soft cap are applied by the register-staged kernel only
+    const bool mod = a.mod.active();
+    if (mod && a.mod.bias_type == FCK_BIAS_ELEMENTWISE) {
+        // an elementwise bias costs a load per score: only the register-staged kernel reads it; ALiBi and the soft cap
+        // are arithmetic on the score and every kernel applies them
         a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
         g_kernel = uniform ? "prefill_kernel<uniform_page,score_mod>" : "prefill_kernel<row_lookup,score_mod>";
         return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }
     if (d <= 128 && q_max_seq_len > 128) {
         a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
-        g_kernel = uniform ? "prefill_pp_kernel<uniform_page>" : "prefill_pp_kernel<row_lookup>";
+        g_kernel = uniform ? (mod ? "prefill_pp_kernel<uniform_page,score_mod>" : "prefill_pp_kernel<uniform_page>")
+                           : (mod ? "prefill_pp_kernel<row_lookup,score_mod>" : "prefill_pp_kernel<row_lookup>");
         return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }
     a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
     if (d == 256 && uniform) {
-        g_kernel = "prefill_dma_kernel<uniform_page>";
+        g_kernel = mod ? "prefill_dma_kernel<uniform_page,score_mod>" : "prefill_dma_kernel<uniform_page>";
         return launch_status(fck::launch_prefill_dma(a, (int)d, dtype, static_cast<hipStream_t>(stream)), what);
+    }
+    if (mod) {
+        g_kernel = uniform ? "prefill_kernel<uniform_page,score_mod>" : "prefill_kernel<row_lookup,score_mod>";
+        return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }
     g_kernel = uniform ? "prefill_kernel<uniform_page>" : "prefill_kernel<row_lookup>";
     return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);

@@ -37,7 +37,8 @@ struct Shape {
 __device__ __forceinline__ int k_swz(int row) { return tiles::k_swz<256>(row); }
 __device__ __forceinline__ int v_swz(int row, int lc) { return tiles::v_swz<256>(row, lc); }
 
-template <typename T, int D>
+// kMod: ALiBi and / or the logits soft cap applied to every score (ArithMod)
+template <typename T, int D, bool kMod = false>
 __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a)
 {
     typedef Shape<D> S;
@@ -91,6 +92,9 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     const bool row_ok = r >= 0 && r < sq_b;
     const int lo_r = row_ok ? mask_lo(mk, r) : 0;
     const int hi_r = row_ok ? mask_hi(mk, r, sk_b) : sk_b;
+    ArithMod amod;
+    if constexpr (kMod) amod.init(a.mod, b, h, row_ok ? r : 0, sq_b, sk_b, a.mask_type, a.window_left, a.window_right);
+    const float scl = kMod ? 1.f : a.scale_log2;  // modified scores come out in the log2 domain already
     // wave-uniform bounds: keys in [w_lo_max, w_hi_min) are visible to every valid row of the wave
     const int wr0 = max(m0 + wave * 32, 0);
     const int wr1 = min(m0 + wave * 32 + 32, sq_b) - 1;
@@ -212,6 +216,12 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
         }
 
         // ---- online softmax (exp2 domain) ---------------------------------------------------------------------
+        if constexpr (kMod) {
+#pragma unroll
+            for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) s[mbk][j] = amod.score(s[mbk][j], kb + mbk * 32 + (j >> 2) * 8 + half * 4 + (j & 3));
+        }
         const bool need_mask = (kb < w_lo_max) || (kb + BN > w_hi_min);
         float tmax = -INFINITY;
         if (need_mask) {
@@ -229,7 +239,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
 #pragma unroll
             for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
         tmax = pair32_max(tmax);
-        tmax *= a.scale_log2;  // scale > 0: max commutes with the scaling
+        tmax *= scl;  // scale > 0: max commutes with the scaling
         // Lazy rescale: the reference m_run only moves when some row's maximum outgrows it by more than kLazy (log2
         // units).  Softmax is shift invariant, so a stale reference is exact; it bounds the exponentials by 2^kLazy.
         constexpr float kLazy = 8.f;
@@ -253,7 +263,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
         for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
-                const float p = fast_exp2(__builtin_fmaf(s[mbk][j], a.scale_log2, -m_ref));
+                const float p = fast_exp2(__builtin_fmaf(s[mbk][j], scl, -m_ref));
                 s[mbk][j] = p;
                 psum += p;
             }
@@ -308,6 +318,10 @@ static hipError_t launch_d(const PrefillArgs& a, hipStream_t st)
     const int g = a.hq / a.hk, gx = (a.batch * a.hk + 7) / 8;
     const dim3 grid(8 * a.m_tiles * gx * g);
     constexpr size_t lds = (size_t)4 * Shape<D>::TILEB + kPrefillPageCache * 4;
+    if (a.mod.active()) {
+        if (a.mod.bias_type == 1) return hipErrorInvalidValue;  // elementwise bias: not in this kernel (the caller routes it away)
+        return launch_with_lds<prefill_dma_kernel<T, D, true>>(grid, dim3(256), lds, st, a);
+    }
     return launch_with_lds<prefill_dma_kernel<T, D>>(grid, dim3(256), lds, st, a);
 }
 

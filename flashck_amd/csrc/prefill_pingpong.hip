@@ -47,7 +47,9 @@ struct PPShape {
 using tiles::k_swz;
 using tiles::v_swz;
 
-template <typename T, int D, int BN, bool kUniformPage>
+// kMod: ALiBi and / or the logits soft cap are applied to every score in the vector phase (ArithMod; an elementwise
+// bias needs a load per score and stays with the register-staged kernel).
+template <typename T, int D, int BN, bool kUniformPage, bool kMod = false>
 __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
 {
     typedef PPShape<D, BN> S;
@@ -109,6 +111,9 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     const bool row_ok = r >= 0 && r < sq_b;
     const int lo_r = row_ok ? mask_lo(mk, r) : 0;
     const int hi_r = row_ok ? mask_hi(mk, r, sk_b) : sk_b;
+    ArithMod amod;
+    if constexpr (kMod) amod.init(a.mod, b, h, row_ok ? r : 0, sq_b, sk_b, a.mask_type, a.window_left, a.window_right);
+    const float scl = kMod ? 1.f : a.scale_log2;  // modified scores come out in the log2 domain already
     // wave-uniform: keys in [w_lo_max, w_hi_min) are visible to every valid row of the wave
     const int wr0 = max(m0 + group * 128 + wg * 32, 0);
     const int wr1 = min(m0 + group * 128 + wg * 32 + 32, sq_b) - 1;
@@ -266,6 +271,12 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     // online softmax of local tile i: s -> pfrag
     auto softmax = [&](int i) __attribute__((always_inline)) {
         const int kb = (t_begin + i) * S::BN;
+        if constexpr (kMod) {
+#pragma unroll
+            for (int mbk = 0; mbk < S::NB; ++mbk)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) s[mbk][j] = amod.score(s[mbk][j], kb + mbk * 32 + (j >> 2) * 8 + half * 4 + (j & 3));
+        }
         const bool need_mask = (kb < w_lo_max) || (kb + S::BN > w_hi_min);
         if (need_mask) {
 #pragma unroll
@@ -283,7 +294,7 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
 #pragma unroll
             for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
         tmax = pair32_max(tmax);
-        tmax *= a.scale_log2;  // scale > 0: max commutes with the scaling
+        tmax *= scl;  // scale > 0: max commutes with the scaling
         // Lazy rescale: the reference m_run only moves when some row's maximum outgrows it by more than kLazy (log2
         // units).  Softmax is shift invariant, so a stale reference is exact; it bounds the exponentials by 2^kLazy.
         constexpr float kLazy = 8.f;
@@ -305,7 +316,7 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
             float p[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                p[e] = fast_exp2(__builtin_fmaf(s[mbk][j0 + e], a.scale_log2, -m_ref));
+                p[e] = fast_exp2(__builtin_fmaf(s[mbk][j0 + e], scl, -m_ref));
                 psum += p[e];
             }
             pfrag[ks4][0] = T::pack2(p[0], p[1]);
@@ -392,6 +403,11 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
     const int g = a.hq / a.hk, gx = (a.batch * a.hk + 7) / 8;
     const dim3 grid(8 * a.m_tiles * gx * g);
     constexpr size_t lds = (size_t)2 * PPShape<D, BN>::RING * PPShape<D, BN>::TILEB + kPrefillPageCache * 4;
+    if (a.mod.active()) {
+        if (a.mod.bias_type == 1) return hipErrorInvalidValue;  // elementwise bias: not in this kernel (the caller routes it away)
+        if (uniform) return launch_with_lds<prefill_pp_kernel<T, D, BN, true, true>>(grid, dim3(512), lds, st, a);
+        return launch_with_lds<prefill_pp_kernel<T, D, BN, false, true>>(grid, dim3(512), lds, st, a);
+    }
     if (uniform) return launch_with_lds<prefill_pp_kernel<T, D, BN, true>>(grid, dim3(512), lds, st, a);
     return launch_with_lds<prefill_pp_kernel<T, D, BN, false>>(grid, dim3(512), lds, st, a);
 }

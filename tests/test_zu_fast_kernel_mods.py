@@ -1,0 +1,82 @@
+"""GPU: ALiBi and the logits soft cap on the direct-to-LDS prefill kernels (long query runs, several key tiles, ragged
+batches, both page addressings), and the column clamp of a narrow elementwise bias."""
+import math
+
+import pytest
+import torch
+
+from flashck_amd import _lib, generators as gen
+from helpers import ATOL, assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _mods(kind, hq, batch, g):
+    if kind == "cap":
+        return dict(logits_soft_cap=2.5)
+    slopes = (torch.rand(batch, hq, generator=g) * 0.2).float() if kind == "alibi_b" else (torch.rand(hq, generator=g) * 0.2).float()
+    kw = dict(alibi_slopes=slopes)
+    if kind == "alibi_cap":
+        kw["logits_soft_cap"] = 3.0
+    return kw
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kind", ["cap", "alibi_h", "alibi_b", "alibi_cap"])
+@pytest.mark.parametrize("d,page,mask", [(128, 128, (2, (-1, 0))), (64, 64, (2, (100, 0))), (128, 48, (2, (-1, 0))), (256, 64, (2, (-1, 0))),
+                                         (256, 128, (1, (-1, 0))), (128, 128, (0, (-1, -1)))])
+def test_batch_prefill_with_arithmetic_modifiers(fmha, orc, dtype, kind, d, page, mask):
+    """Sequences of 300 / 700 / 129 / 1 tokens: up to 3 row tiles and 11 key tiles per workgroup; page 48 takes the per-row
+    lookup variant of the ping-pong kernel."""
+    g = torch.Generator().manual_seed(7 + d + page)
+    w = gen.workload_varlen_prefill(seed=40 + d + page, batch=4, hq=4, hk=2, head_dim=d, page_size=page, dtype=dtype, lens=[300, 700, 129, 1])
+    kw = _mods(kind, 4, 4, g)
+    a = [dev(w[k]) for k in ("q", "k_cache", "v_cache", "cu_seqlens_q", "kv_indptr", "kv_page_indices", "kv_last_page_lens")]
+    o = fmha.fmha_batch_prefill(*a, max_seqlen_q=w["max_seqlen_q"], scale=w["scale"], mask_type=mask[0], window=mask[1],
+                                **{k: dev(v) for k, v in kw.items()})
+    name = _lib.load().fck_fmha_last_kernel()
+    if d == 256:
+        assert name == b"prefill_dma_kernel<uniform_page,score_mod>"
+    else:
+        assert name == (b"prefill_pp_kernel<uniform_page,score_mod>" if page % 64 == 0 else b"prefill_pp_kernel<row_lookup,score_mod>")
+    ro = orc.fmha_fwd(w["q"], w["k_cache"], w["v_cache"], seqstart_q=w["cu_seqlens_q"], kv_indptr=w["kv_indptr"],
+                      kv_page_indices=w["kv_page_indices"], kv_last_page_lens=w["kv_last_page_lens"], scale=w["scale"], mask_type=mask[0],
+                      window=mask[1], **kw)
+    assert_close(o, ro, ATOL[dtype], f"{kind} on {name.decode()}")
+
+
+def test_pagedkv_batch_mode_with_alibi_on_the_fast_kernel(fmha, orc):
+    g = torch.Generator().manual_seed(23)
+    dtype, hq, hk, d, sq = torch.bfloat16, 8, 2, 128, 260
+    kv = gen.paged_kv([260, 400], hk, d, dtype, g, 128)
+    q = gen.randn((2, sq, hq, d), dtype, g)
+    slopes = (torch.rand(2, hq, generator=g) * 0.3).float()
+    o = fmha.fmha_fwd_pagedkv(dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]), dev(kv["seqlen_k"]), dev(kv["block_table"]), mask_type=2,
+                              window=(-1, 0), alibi_slopes=dev(slopes))
+    assert _lib.load().fck_fmha_last_kernel() == b"prefill_pp_kernel<uniform_page,score_mod>"
+    ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], mask_type=2, window=(-1, 0),
+                      alibi_slopes=slopes)
+    assert_close(o, ro, 2e-2, "paged prefill with ALiBi")
+
+
+@pytest.mark.parametrize("path", ["decode", "prefill"])
+def test_narrow_bias_is_clamped_to_its_last_column(fmha, orc, path):
+    """A bias with fewer columns than a sequence has keys: reads are clamped to the last column (never out of bounds);
+    the oracle gets the same bias widened by repeating that column."""
+    g = torch.Generator().manual_seed(29)
+    dtype, hq, hk, d = torch.bfloat16, 4, 2, 128
+    lens = [90, 200]
+    kv = gen.paged_kv(lens, hk, d, dtype, g, 64)
+    sq = 1 if path == "decode" else 40
+    cols = 120                                    # sequence 1 has 200 keys
+    q = gen.randn((2, sq, hq, d), dtype, g)
+    bias = gen.randn((2, hq, sq, cols), dtype, g)
+    wide = torch.cat([bias, bias[..., -1:].expand(2, hq, sq, 200 - cols)], dim=-1).contiguous()
+    args = (dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]))
+    if path == "decode":
+        o = fmha.fmha_decode_paged(*args, dev(kv["seqlen_k"]), dev(kv["block_table"]), num_splits=2, bias=dev(bias))
+    else:
+        o = fmha.fmha_fwd_pagedkv(*args, dev(kv["seqlen_k"]), dev(kv["block_table"]), mask_type=2, window=(-1, 0), bias=dev(bias))
+    ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqlen_k=kv["seqlen_k"], block_table=kv["block_table"],
+                      mask_type=0 if path == "decode" else 2, window=(-1, -1) if path == "decode" else (-1, 0), bias=wide)
+    assert_close(o, ro, 2e-2, f"narrow bias, {path}")
