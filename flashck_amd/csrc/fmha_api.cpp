@@ -78,6 +78,17 @@ int fill_kv8(fck::PrefillArgs& a, const fck_fmha_attrs* at, int64_t d, int64_t d
     return FCK_OK;
 }
 
+// tile variant of a prefill call (range only; whether the problem can take it is decided where the kernel is chosen)
+int fill_variant(fck::PrefillArgs& a, const fck_fmha_attrs* at)
+{
+    a.variant = 0;
+    if (!at || at->prefill_variant == 0) return FCK_OK;
+    if (at->prefill_variant < 1 || at->prefill_variant > 4)
+        return fail(FCK_ERR_INVALID_ARGUMENT, "prefill_variant %d out of range [0,4]", at->prefill_variant);
+    a.variant = at->prefill_variant;
+    return FCK_OK;
+}
+
 // Bias / ALiBi / soft cap of a call: `bias` is the positional pointer of the entry points that have one (else null).
 
 int fill_mod(fck::ScoreMod& m, const void* bias, const fck_fmha_attrs* at, float scale, uint32_t mask_type, int64_t hq)
@@ -540,6 +551,11 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t
     // takes the 4-wave kernel that sends K/V tiles straight to LDS (128 rows per workgroup) when a 64-key tile never
     // straddles a page; short runs at head dim <= 128 and page sizes that are not a multiple of 64 take the 4-wave
     // kernel that stages K/V through registers.
+    // Tile variants (2..4) exist for the plain ping-pong kernel on uniform pages; variant 1 names the default schedule of
+    // whatever kernel the call takes.
+    if (a.variant > 1 && !(d_qk == d && dv == d && d <= 128 && q_max_seq_len > 128 && uniform && !a.mod.active() && !a.kv8))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "prefill_variant %d needs the ping-pong kernel: head dim 64 or 128, query runs longer than 128, "
+                                              "pages a multiple of 64 (or no pages), no bias / ALiBi / soft cap / fp8 cache", a.variant);
     if (d_qk != d || dv != d) {
         // head dims other than 64 / 128 / 256, or qk_head_dim != v_head_dim: the register-staged kernel pads them
         a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
@@ -562,7 +578,10 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t
     }
     if (d <= 128 && q_max_seq_len > 128) {
         a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
-        g_kernel = uniform ? (mod ? "prefill_pp_kernel<uniform_page,score_mod>" : "prefill_pp_kernel<uniform_page>")
+        static const char* const variants[5] = {"prefill_pp_kernel<uniform_page>", "prefill_pp_kernel<uniform_page>",
+                                                "prefill_pp_kernel<uniform_page,fast_requests>", "prefill_pp_kernel<uniform_page,max_in_matrix_phase>",
+                                                "prefill_pp_kernel<uniform_page,fast_requests,max_in_matrix_phase>"};
+        g_kernel = uniform ? (mod ? "prefill_pp_kernel<uniform_page,score_mod>" : variants[a.variant])
                            : (mod ? "prefill_pp_kernel<row_lookup,score_mod>" : "prefill_pp_kernel<row_lookup>");
         return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }
@@ -616,6 +635,7 @@ int fck_fmha_fwd_attrs(const void* q, const void* k, const void* v, const void* 
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
     if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
+    if (int rc = fill_variant(a, attrs)) return rc;
     a.kv.page_shift = -1;
     a.kv.seqlen_k_ptr = seqlen_k_ptr;  // group mode: logical key counts of padded packed sequences
     if (seqstart_q) {
@@ -670,6 +690,7 @@ int fck_fmha_batch_prefill_attrs(const void* q, const void* k_cache, const void*
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
     if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
+    if (int rc = fill_variant(a, attrs)) return rc;
     a.kv.mode = 3;
     a.kv.kv_indptr = kv_indptr;
     a.kv.kv_page_indices = kv_page_indices;
@@ -723,6 +744,7 @@ int fck_fmha_fwd_pagedkv_attrs(const void* q, const void* k_cache, const void* v
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
     if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
+    if (int rc = fill_variant(a, attrs)) return rc;
     a.kv.mode = 2;
     a.kv.block_table = block_table;
     a.kv.block_table_stride = (int32_t)batch_stride_block_table;

@@ -96,6 +96,7 @@ struct PrefillArgs {
     int64_t window_left, window_right;
     ScoreMod mod;  // bias / ALiBi / soft cap; all zero: none (an elementwise bias only in the 4-wave kernel of prefill.hip)
     int32_t d, dv;  // head dims of Q/K and of V/O as stored; other than the kernel's D only in the 4-wave kernel of prefill.hip
+    int32_t variant;  // tile variant of the ping-pong kernel: 0 / 1 the default schedule, 2..4 see prefill_pingpong.hip
     int32_t kv8;      // K and V are fp8 (e4m3); the K scale is folded into scale_log2 / mod.scale by the caller (4-wave kernel only)
     float v_descale;  // factor on the output (1 unless V is quantised)
 };

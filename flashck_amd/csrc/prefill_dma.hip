@@ -94,7 +94,6 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     const int hi_r = row_ok ? mask_hi(mk, r, sk_b) : sk_b;
     ArithMod amod;
     if constexpr (kMod) amod.init(a.mod, b, h, row_ok ? r : 0, sq_b, sk_b, a.mask_type, a.window_left, a.window_right);
-    const float scl = kMod ? 1.f : a.scale_log2;  // modified scores come out in the log2 domain already
     // wave-uniform bounds: keys in [w_lo_max, w_hi_min) are visible to every valid row of the wave
     const int wr0 = max(m0 + wave * 32, 0);
     const int wr1 = min(m0 + wave * 32 + 32, sq_b) - 1;
@@ -239,7 +238,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
 #pragma unroll
             for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
         tmax = pair32_max(tmax);
-        tmax *= scl;  // scale > 0: max commutes with the scaling
+        if constexpr (!kMod) tmax *= a.scale_log2;  // scale > 0: max commutes with the scaling (modified scores are in the log2 domain already)
         // Lazy rescale: the reference m_run only moves when some row's maximum outgrows it by more than kLazy (log2
         // units).  Softmax is shift invariant, so a stale reference is exact; it bounds the exponentials by 2^kLazy.
         constexpr float kLazy = 8.f;
@@ -263,7 +262,7 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
         for (int mbk = 0; mbk < 2; ++mbk)
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
-                const float p = fast_exp2(__builtin_fmaf(s[mbk][j], scl, -m_ref));
+                const float p = kMod ? fast_exp2(s[mbk][j] - m_ref) : fast_exp2(__builtin_fmaf(s[mbk][j], a.scale_log2, -m_ref));
                 s[mbk][j] = p;
                 psum += p;
             }

@@ -49,9 +49,16 @@ using tiles::v_swz;
 
 // kMod: ALiBi and / or the logits soft cap are applied to every score in the vector phase (ArithMod; an elementwise
 // bias needs a load per score and stays with the register-staged kernel).
-template <typename T, int D, int BN, bool kUniformPage, bool kMod = false>
+// kVar: tile variants a tuner can choose between (fck_fmha_attrs.prefill_variant - 1; 0 is the default schedule):
+//   bit 0  requests of a tile whose 64 rows all exist use byte offsets computed once per workgroup (no clamp and no
+//          multiply per request; the scalar base carries the tile)
+//   bit 1  the per-lane maximum of a tile's raw scores is taken at the end of the matrix phase that produced them,
+//          which shortens the (longer) vector phase by that much; tiles that need masking take it again after the mask
+template <typename T, int D, int BN, bool kUniformPage, bool kMod = false, int kVar = 0>
 __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
 {
+    constexpr bool kFastRequests = (kVar & 1) != 0, kMaxInMatrixPhase = (kVar & 2) != 0;
+    static_assert(kVar == 0 || (kUniformPage && !kMod), "tile variants exist for the plain uniform-page kernel");
     typedef PPShape<D, BN> S;
     typedef typename T::vec8 vec8;
     static_assert(S::NB == 2, "the matrix phase is written for 64-key tiles");
@@ -113,7 +120,6 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     const int hi_r = row_ok ? mask_hi(mk, r, sk_b) : sk_b;
     ArithMod amod;
     if constexpr (kMod) amod.init(a.mod, b, h, row_ok ? r : 0, sq_b, sk_b, a.mask_type, a.window_left, a.window_right);
-    const float scl = kMod ? 1.f : a.scale_log2;  // modified scores come out in the log2 domain already
     // wave-uniform: keys in [w_lo_max, w_hi_min) are visible to every valid row of the wave
     const int wr0 = max(m0 + group * 128 + wg * 32, 0);
     const int wr1 = min(m0 + group * 128 + wg * 32 + 32, sq_b) - 1;
@@ -145,6 +151,7 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     float m_run = -INFINITY, l_run = 0.f;
     f32x16_t s[S::NB];          // scores of the tile between its M and V phase
     u32x4_t pfrag[2 * S::NB];   // probabilities of the tile between its V phase and the next M phase
+    float tmax_pre = -INFINITY;  // kMaxInMatrixPhase: per-lane maximum of s, from the matrix phase that produced it
 
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k);
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v);
@@ -165,6 +172,16 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         cp_v[u] = tiles::v_chunk_at<D>(row, pc) * 8;
     }
 
+    // kFastRequests: byte offsets of a whole tile's requests
+    uint32_t cp_koff[S::LD], cp_voff[S::LD];
+    if constexpr (kFastRequests) {
+#pragma unroll
+        for (int u = 0; u < S::LD; ++u) {
+            cp_koff[u] = (uint32_t)(cp_row[u] * (int)row_stride + cp_k[u]) * 2u;
+            cp_voff[u] = (uint32_t)(cp_row[u] * (int)row_stride + cp_v[u]) * 2u;
+        }
+    }
+
     // First cache row of every tile (uniform-page path), cached per workgroup (see tiles::FirstRows)
     tiles::FirstRows<S::BN> first_rows{(int FCK_LDS*)(lds + 2 * kRing * S::TILEB)};
     if constexpr (kUniformPage) first_rows.fill(a.kv, ks, t_begin, n, tid, 512);
@@ -172,7 +189,8 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     auto tile = [&](int i) __attribute__((always_inline)) { return min(i, n - 1); };  // requests past the end re-read the last tile
     // request this wave's share of local tile `want` into ring buffer want % kRing (past the last tile: that tile
     // again); row0 = tile_row0(tile(want)) on the uniform-page path
-    auto request = [&](const uint16_t* base, char FCK_LDS* ring, int want, int64_t row0, const int (&cp_c)[S::LD]) __attribute__((always_inline)) {
+    auto request = [&](const uint16_t* base, char FCK_LDS* ring, int want, int64_t row0, const int (&cp_c)[S::LD],
+                       const uint32_t (&cp_off)[S::LD]) __attribute__((always_inline)) {
         const int i = tile(want);
         const int kb = (t_begin + i) * S::BN;
         const int room = last_key - kb;
@@ -183,7 +201,10 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
             const uint32_t dst = lds_address(ring + slot_ * S::TILEB + (wave + 8 * u) * 1024);
             if constexpr (kUniformPage) {
                 const uint16_t* tb = base + (row0 * row_stride + hkv * D);
-                tiles::load_to_lds(dst, tb, (uint32_t)(row * (int)row_stride + cp_c[u]) * 2u);
+                if (kFastRequests && room >= S::BN - 1)
+                    tiles::load_to_lds(dst, tb, cp_off[u]);
+                else
+                    tiles::load_to_lds(dst, tb, (uint32_t)(row * (int)row_stride + cp_c[u]) * 2u);
             } else {
                 tiles::load_to_lds(dst, base + kv_row(a.kv, ks, kb + row) * row_stride + hkv * D + cp_c[u]);
             }
@@ -266,6 +287,15 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);
+        if constexpr (kMaxInMatrixPhase && kQk) {
+            float t = s[0][0];
+#pragma unroll
+            for (int mbk = 0; mbk < S::NB; ++mbk)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) t = fmaxf(t, s[mbk][j]);
+            FCK_PIN_VGPR(t);  // stays in this phase
+            tmax_pre = t;
+        }
     };
 
     // online softmax of local tile i: s -> pfrag
@@ -289,12 +319,16 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
                 }
         }
         float tmax = -INFINITY;
+        if (kMaxInMatrixPhase && !need_mask) {
+            tmax = tmax_pre;
+        } else {
 #pragma unroll
-        for (int mbk = 0; mbk < S::NB; ++mbk)
+            for (int mbk = 0; mbk < S::NB; ++mbk)
 #pragma unroll
-            for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
+                for (int j = 0; j < 16; ++j) tmax = fmaxf(tmax, s[mbk][j]);
+        }
         tmax = pair32_max(tmax);
-        tmax *= scl;  // scale > 0: max commutes with the scaling
+        if constexpr (!kMod) tmax *= a.scale_log2;  // scale > 0: max commutes with the scaling (modified scores are in the log2 domain already)
         // Lazy rescale: the reference m_run only moves when some row's maximum outgrows it by more than kLazy (log2
         // units).  Softmax is shift invariant, so a stale reference is exact; it bounds the exponentials by 2^kLazy.
         constexpr float kLazy = 8.f;
@@ -316,7 +350,10 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
             float p[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                p[e] = fast_exp2(__builtin_fmaf(s[mbk][j0 + e], scl, -m_ref));
+                if constexpr (kMod)
+                    p[e] = fast_exp2(s[mbk][j0 + e] - m_ref);
+                else
+                    p[e] = fast_exp2(__builtin_fmaf(s[mbk][j0 + e], a.scale_log2, -m_ref));
                 psum += p[e];
             }
             pfrag[ks4][0] = T::pack2(p[0], p[1]);
@@ -348,11 +385,11 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
             r1 = tile_row0(tile(1));
             r2 = tile_row0(tile(2));
         }
-        request(kp, k_ring, 0, r0, cp_k);
-        request(vp, v_ring, 0, r0, cp_v);
-        request(kp, k_ring, 1, r1, cp_k);
-        request(kp, k_ring, 2, r2, cp_k);  // batch -1
-        request(vp, v_ring, 1, r1, cp_v);
+        request(kp, k_ring, 0, r0, cp_k, cp_koff);
+        request(vp, v_ring, 0, r0, cp_v, cp_voff);
+        request(kp, k_ring, 1, r1, cp_k, cp_koff);
+        request(kp, k_ring, 2, r2, cp_k, cp_koff);  // batch -1
+        request(vp, v_ring, 1, r1, cp_v, cp_voff);
         wait_vm(KeepBatch{});
         __syncthreads();
         if (group == 1) __syncthreads();  // skew: group 1 idles through phase 0
@@ -362,8 +399,8 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         for (int i = 0; i + 1 < n; ++i) {
             int64_t row_k = 0;
             if constexpr (kUniformPage) row_k = tile_row0(tile(i + 3));
-            request(kp, k_ring, i + 3, row_k, cp_k);
-            request(vp, v_ring, i + 2, row_v, cp_v);
+            request(kp, k_ring, i + 3, row_k, cp_k, cp_koff);
+            request(vp, v_ring, i + 2, row_v, cp_v, cp_voff);
             row_v = row_k;
             softmax(i);
             __syncthreads();
@@ -407,6 +444,16 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
         if (a.mod.bias_type == 1) return hipErrorInvalidValue;  // elementwise bias: not in this kernel (the caller routes it away)
         if (uniform) return launch_with_lds<prefill_pp_kernel<T, D, BN, true, true>>(grid, dim3(512), lds, st, a);
         return launch_with_lds<prefill_pp_kernel<T, D, BN, false, true>>(grid, dim3(512), lds, st, a);
+    }
+    if (a.variant > 0) {  // validated by the caller: plain call, uniform pages, variant in [1, 4]
+        if (!uniform) return hipErrorInvalidValue;
+        switch (a.variant) {
+        case 1: break;  // the default schedule, by name
+        case 2: return launch_with_lds<prefill_pp_kernel<T, D, BN, true, false, 1>>(grid, dim3(512), lds, st, a);
+        case 3: return launch_with_lds<prefill_pp_kernel<T, D, BN, true, false, 2>>(grid, dim3(512), lds, st, a);
+        case 4: return launch_with_lds<prefill_pp_kernel<T, D, BN, true, false, 3>>(grid, dim3(512), lds, st, a);
+        default: return hipErrorInvalidValue;
+        }
     }
     if (uniform) return launch_with_lds<prefill_pp_kernel<T, D, BN, true>>(grid, dim3(512), lds, st, a);
     return launch_with_lds<prefill_pp_kernel<T, D, BN, false>>(grid, dim3(512), lds, st, a);

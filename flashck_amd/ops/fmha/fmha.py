@@ -25,7 +25,7 @@ __all__ = [
     "ROPE_HALF_ROTATED", "fmha_fwd", "fmha_fwd_varlen", "fmha_fwd_splitkv", "fmha_fwd_splitkv_combine",
     "fmha_fwd_splitkv_fused", "fused_splitkv_fits",
     "fmha_fwd_appendkv", "fmha_batch_prefill", "fmha_fwd_pagedkv", "fmha_decode_paged", "fmha_decode_step",
-    "tune_decode_num_splits", "DecodeWorkspace", "num_splits_heuristic", "splitkv_workspace", "validate_paged", "fused_reset",
+    "tune_decode_num_splits", "tune_prefill_variant", "DecodeWorkspace", "num_splits_heuristic", "splitkv_workspace", "validate_paged", "fused_reset",
 ]
 
 # GenericAttentionMaskEnum / RopeEnum, core/profiling/attention/fmha_library.h:81-87,195-200
@@ -123,7 +123,7 @@ def _window(window):
 
 
 def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols, kv_fp8=False, k_descale=1.0, v_descale=1.0,
-           decode_variant=0):
+           decode_variant=0, prefill_variant=0):
     """fck_fmha_attrs for a call, or None when no score modifier is asked for.
 
     bias (elementwise, BiasEnum ELEMENTWISE_BIAS): q's dtype, last dim contiguous; batch mode [1|B, 1|Hq, sq, >= sk],
@@ -135,7 +135,9 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
         raise ValueError("logits_soft_cap must be finite and >= 0")
     if int(decode_variant) not in (0, 1, 2):
         raise ValueError("decode_variant must be 0 (library's choice), 1 (one KV head per workgroup) or 2 (head pairs)")
-    if bias is None and alibi_slopes is None and cap == 0.0 and not kv_fp8 and not decode_variant:
+    if int(prefill_variant) not in (0, 1, 2, 3, 4):
+        raise ValueError("prefill_variant must be 0 (library's choice) or 1..4 (see fck_fmha_attrs.prefill_variant)")
+    if bias is None and alibi_slopes is None and cap == 0.0 and not kv_fp8 and not decode_variant and not prefill_variant:
         return None, None
     if bias is not None and alibi_slopes is not None:
         raise ValueError("bias and alibi_slopes are exclusive (one BiasEnum per call)")
@@ -143,6 +145,7 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
     a.size = ctypes.sizeof(_lib.Attrs)
     a.logits_soft_cap = cap
     a.decode_variant = int(decode_variant)
+    a.prefill_variant = int(prefill_variant)
     if kv_fp8:
         if not (float(k_descale) > 0.0 and float(v_descale) > 0.0 and math.isfinite(k_descale) and math.isfinite(v_descale)):
             raise ValueError("k_descale and v_descale must be positive and finite")
@@ -532,10 +535,38 @@ def fmha_fwd_appendkv(q, k_cache, v_cache, knew, vnew, seqlen_k, *, cu_seqlens_k
         _call("fck_fmha_fwd_appendkv", *args, _stream())
 
 
+def _usable_prefill_variant(variant, head_dim, v_head_dim, max_seqlen_q, page_size):
+    """A cached tile variant is a hint (the problem class is coarser than the variant's preconditions): variants 2..4
+    need the ping-pong kernel, i.e. equal head dims of 64 or 128, query runs longer than 128 and pages a multiple of 64."""
+    variant = int(variant)
+    if variant in (2, 3, 4):
+        ok = head_dim == v_head_dim and head_dim in (64, 128) and max_seqlen_q > 128 and page_size % 64 == 0
+        return variant if ok else 0
+    return variant if variant == 1 else 0
+
+
+def tune_prefill_variant(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_indices, kv_last_page_lens=None, *, max_seqlen_q: int,
+                         variants=(1, 2, 3, 4), cache=None, **kwargs) -> dict:
+    """Time fmha_batch_prefill with each tile variant on these tensors and record the fastest for the problem class (see
+    utils/tuning.py); later calls on problems of that class with prefill_variant = 0 use it.  Returns the record."""
+    tq, Hq, D = q.shape
+    _, page, Hk, Dv = v_cache.shape
+    mask_type = kwargs.get("mask_type", MASK_BOTTOM_RIGHT)
+    problem = tuning.prefill_problem(Hq, Hk, D, max_seqlen_q, tq, page, "fp16" if q.dtype == torch.float16 else "bf16", mask_type)
+    out = torch.empty(tq, Hq, Dv, dtype=q.dtype, device=q.device)
+
+    def run(variant):
+        fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_indices, kv_last_page_lens, max_seqlen_q=max_seqlen_q,
+                           out=out, prefill_variant=variant, **kwargs)
+        return _lib.load().fck_fmha_last_kernel().decode()
+
+    return tuning.tune_prefill_variant(run, tuning.gpu_timer, variants, problem, cache=cache)
+
+
 def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_indices, kv_last_page_lens=None, *,
                        max_seqlen_q: int, scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0),
                        out=None, bias=None, alibi_slopes=None, logits_soft_cap: float = 0.0, k_descale: float = 1.0,
-                       v_descale: float = 1.0) -> torch.Tensor:
+                       v_descale: float = 1.0, prefill_variant: int = 0) -> torch.Tensor:
     """Varlen prefill over a page list: q [total_q,Hq,D]; sequence b owns pages
     kv_page_indices[kv_indptr[b]:kv_indptr[b+1]] of the cache [num_pages, page_size, Hk, D].  The caches may be
     torch.float8_e4m3fn with the static scales k_descale / v_descale (value = descale * stored)."""
@@ -558,7 +589,12 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
     wl, wr = _window(window)
     _debug_validate(kv_indptr=kv_indptr, kv_page_indices=kv_page_indices, kv_last_page_lens=kv_last_page_lens,
                     num_total_pages=num_pages, page_size=page)
-    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1, kv_fp8, k_descale, v_descale)
+    plain = bias is None and alibi_slopes is None and not logits_soft_cap and not kv_fp8
+    if not prefill_variant and plain:   # a tuned tile variant for this class of problems, if one is recorded and fits
+        prefill_variant = _usable_prefill_variant(tuning.choose_prefill_variant(tuning.prefill_problem(
+            Hq, Hk, D, max_seqlen_q, tq, page, "fp16" if q.dtype == torch.float16 else "bf16", mask_type)), D, Dv, max_seqlen_q, page)
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1, kv_fp8, k_descale, v_descale,
+                      prefill_variant=prefill_variant)
     if at is None:
         _call("fck_fmha_batch_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
               _ptr(kv_page_indices), _ptr(kv_last_page_lens), num_pages, page, B, Hq, Hk, D, Dv, max_seqlen_q,
@@ -573,7 +609,8 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
 
 def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q=None, max_seqlen_q: int = 0,
                      scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0), out=None, bias=None,
-                     alibi_slopes=None, logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0) -> torch.Tensor:
+                     alibi_slopes=None, logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0,
+                     prefill_variant: int = 0) -> torch.Tensor:
     """Prefill over a block table (no splits): q [B,sq,Hq,D] or packed [total_q,Hq,D].  The caches may be
     torch.float8_e4m3fn with the static scales k_descale / v_descale (value = descale * stored)."""
     group = cu_seqlens_q is not None
@@ -598,7 +635,8 @@ def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q
     o = _out("out", out, (*q.shape[:-1], Dv), q.dtype, q)
     wl, wr = _window(window)
     _debug_validate(seqlen_k=seqlen_k, block_table=block_table, num_total_pages=k_cache.shape[0], page_size=page)
-    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, q.shape[0] if group else sq, 1, kv_fp8, k_descale, v_descale)
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, q.shape[0] if group else sq, 1, kv_fp8, k_descale, v_descale,
+                      prefill_variant=prefill_variant)
     if at is None:
         _call("fck_fmha_fwd_pagedkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
               _ptr(block_table), block_table.shape[1], page, B, sq, Hq, Hk, D, Dv, max_seqlen_q or sq, _scale(scale, D), wl, wr,

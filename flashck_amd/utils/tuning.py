@@ -18,7 +18,7 @@ from typing import Callable, Dict, Iterable, Optional
 from . import flags
 
 __all__ = ["TuningCache", "default_cache", "splitkv_problem", "choose_num_splits", "choose_splitkv", "tune_num_splits",
-           "environment"]
+           "prefill_problem", "choose_prefill_variant", "tune_prefill_variant", "environment"]
 
 FILE_NAME = "flashck_amd_tuning.json"
 SCHEMA = 1
@@ -192,6 +192,59 @@ def tune_num_splits(run: Callable[..., Optional[str]], timer: Callable[[Callable
     if nbytes:
         rec["bandwidth_gbs"] = nbytes / best[1] / 1e9
     cache.insert(SPLITKV, problem, rec)
+    return rec
+
+
+PREFILL = "fmha_fwd_prefill"
+
+
+def prefill_problem(q_num_heads, kv_num_heads, head_dim, max_seqlen_q, total_q, page_size=0, dtype="bf16", mask_type=2) -> str:
+    """Key of a prefill problem class: exact head geometry and mask type, power-of-two buckets for the longest query run
+    and the packed query rows."""
+    return (f"dtype={dtype},hq={int(q_num_heads)},hk={int(kv_num_heads)},d={int(head_dim)},page={int(page_size)},mask={int(mask_type)},"
+            f"sq<={_bucket_pow2(max_seqlen_q)},tq<={_bucket_pow2(total_q)}")
+
+
+def choose_prefill_variant(problem: str, cache: Optional[TuningCache] = None) -> int:
+    """Tile variant recorded for the problem class when tuning is on, else 0 (the library's choice)."""
+    if flags.flag("FC_TUNING_MODE") != 0:
+        rec = (cache or default_cache()).query(PREFILL, problem)
+        if rec is not None and 0 <= int(rec.get("variant", 0)) <= 4:
+            return int(rec["variant"])
+    return 0
+
+
+def tune_prefill_variant(run: Callable[[int], Optional[str]], timer: Callable[[Callable[[], None], int, int], float],
+                         variants: Iterable[int], problem: str, flops: int = 0, cache: Optional[TuningCache] = None) -> dict:
+    """Measure `run(variant)` for every tile variant and record the fastest for `problem` - the (shape -> tile instance)
+    half of what ProfilingDB keeps (core/profiling/profiling_db.cc:64-71).  A variant the problem cannot take (run raises
+    ValueError / NotImplementedError) is skipped.  An existing record is kept unless FC_FORCE_PROFILING is set."""
+    cache = cache or default_cache()
+    if not flags.flag("FC_FORCE_PROFILING"):
+        rec = cache.query(PREFILL, problem)
+        if rec is not None:
+            return rec
+    cold, repeats = flags.flag("FC_TUNING_NUM_COLD_ITERATION"), flags.flag("FC_TUNING_NUM_REPEATS")
+    best, tried = None, {}
+    for variant in sorted(set(int(v) for v in variants)):
+        names = []
+        try:
+            t = float(timer(lambda v=variant: names.append(run(v)), cold, repeats))
+        except (ValueError, NotImplementedError):
+            continue
+        tried[f"v{variant}"] = t * 1e6
+        if flags.flag("FC_TUNING_LOG"):
+            print(f"[flashck tuning] {problem}: prefill_variant={variant} {t * 1e6:.1f} us")
+        if best is None or t < best[1]:
+            best = (variant, t, names[-1] if names else None)
+    if best is None:
+        raise ValueError("no prefill variant this problem can take")
+    rec = {"variant": best[0], "latency_us": best[1] * 1e6, "tried_us": tried}
+    if isinstance(best[2], str):
+        rec["kernel"] = best[2]
+    if flops:
+        rec["tflops"] = flops / best[1] / 1e12
+    cache.insert(PREFILL, problem, rec)
     return rec
 
 

@@ -95,8 +95,12 @@ typedef struct fck_fmha_attrs {
      * 2 = two adjacent KV heads per workgroup (16-key tiles, 512-byte row pieces; needs an even kv_num_heads, at most
      * 16 packed query rows, head dim <= 128 and no bias / soft cap).  A variant the problem cannot take is an error. */
     int32_t decode_variant;
-    /* Prefill kernel variant, likewise: 0 = the library chooses; see fck_fmha_fwd for the values.  A variant the problem
-     * cannot take is an error. */
+    /* Prefill tile variant, likewise: 0 = the library chooses; 1 = the default schedule of the kernel the call takes;
+     * 2..4 = variants of the 8-wave ping-pong kernel (2: byte offsets of whole-tile requests computed once per
+     * workgroup; 3: a tile's row maximum taken in the matrix phase that produced its scores; 4: both), which need head
+     * dim 64 or 128, query runs longer than 128 rows, pages a multiple of 64 keys (or an unpaged cache) and no bias /
+     * ALiBi / soft cap / fp8 cache.  A variant the problem cannot take is an error.  All variants give the same
+     * results up to the rounding of the running maximum. */
     int32_t prefill_variant;
     /* ELEMENTWISE_BIAS: columns a bias row holds.  A key index is clamped to the last of them before the bias is read,
      * so a bias narrower than a sequence's key count is never read out of bounds (the scores of such keys then use

@@ -214,3 +214,34 @@ def test_decode_step_drops_a_cached_variant_it_cannot_take(monkeypatch, tmp_path
         kc = torch.zeros(4, 128, 8, 128, dtype=torch.bfloat16)
         F.fmha_decode_step(q, kn, kn, kc, kc, torch.tensor([5, 9], dtype=torch.int32), torch.tensor([[0, 1], [2, 3]], dtype=torch.int32))
         assert seen[-1] == (3, want), (n, seen[-1])
+
+
+def test_prefill_variant_tuner_and_lookup(tmp_path):
+    c = tuning.TuningCache(str(tmp_path), ENV)
+    cost = {1: 3e-3, 2: 2.5e-3, 3: None, 4: 2.8e-3}   # variant 3 is refused
+    ran = []
+
+    def run(v):
+        if cost[v] is None:
+            raise ValueError("cannot take it")
+        ran.append(v)
+        return f"kernel<v{v}>"
+
+    def timer(fn, cold, repeats):
+        fn()
+        return cost[ran[-1]]
+
+    problem = tuning.prefill_problem(32, 8, 128, 8000, 66000, 128, "bf16", 2)
+    assert tuning.choose_prefill_variant(problem, cache=c) == 0
+    rec = tuning.tune_prefill_variant(run, timer, (1, 2, 3, 4), problem, flops=int(1.7e12), cache=c)
+    assert rec["variant"] == 2 and rec["kernel"] == "kernel<v2>" and set(rec["tried_us"]) == {"v1", "v2", "v4"} and abs(rec["tflops"] - 680.0) < 1e-6
+    assert tuning.choose_prefill_variant(problem, cache=c) == 2
+    assert tuning.choose_prefill_variant(tuning.prefill_problem(32, 8, 128, 8000, 66000, 128, "bf16", 0), cache=c) == 0   # another mask: another class
+    assert tuning.prefill_problem(32, 8, 128, 8192, 65536, 128) == tuning.prefill_problem(32, 8, 128, 5000, 40000, 128)  # buckets
+    flags.set_flag_value("FC_TUNING_MODE", "0")
+    assert tuning.choose_prefill_variant(problem, cache=c) == 0
+    flags.set_flag_value("FC_TUNING_MODE", "2")
+    from flashck_amd.ops.fmha import fmha as F
+    assert F._usable_prefill_variant(3, 128, 128, 300, 128) == 3 and F._usable_prefill_variant(3, 128, 128, 300, 0) == 3
+    assert F._usable_prefill_variant(3, 256, 256, 300, 128) == 0 and F._usable_prefill_variant(2, 128, 128, 128, 128) == 0
+    assert F._usable_prefill_variant(4, 128, 128, 300, 48) == 0 and F._usable_prefill_variant(1, 256, 64, 1, 7) == 1
