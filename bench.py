@@ -179,16 +179,24 @@ def bench_decode(args, torch, fmha, gen, which):
     return res
 
 
-def bench_prefill(args, torch, fmha, gen, d, steps, warmup):
+def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=False, kv_fp8=False):
+    """variant: tile variant (fck_fmha_attrs.prefill_variant); alibi: with per-head ALiBi slopes; kv_fp8: K/V cache as e4m3"""
     w = gen.workload_varlen_prefill(head_dim=d)
     dev = "cuda"
+    kw = {}
+    if alibi:
+        kw["alibi_slopes"] = (torch.arange(1, 33, dtype=torch.float32) / 256).to(dev)
+    if kv_fp8:
+        w["k_cache"] = (w["k_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
+        w["v_cache"] = (w["v_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
+        kw.update(k_descale=0.0625, v_descale=0.0625)
     a = [w[k].to(dev) for k in ("q", "k_cache", "v_cache", "cu_seqlens_q", "kv_indptr", "kv_page_indices", "kv_last_page_lens")]
     o = torch.empty_like(a[0])
 
     def step(i, ev):
         if ev is not None:
             ev[0].record()
-        fmha.fmha_batch_prefill(*a, max_seqlen_q=w["max_seqlen_q"], scale=w["scale"], out=o)
+        fmha.fmha_batch_prefill(*a, max_seqlen_q=w["max_seqlen_q"], scale=w["scale"], out=o, prefill_variant=variant, **kw)
         if ev is not None:
             ev[1].record()
 
@@ -198,7 +206,8 @@ def bench_prefill(args, torch, fmha, gen, d, steps, warmup):
     flops = gen.prefill_flops(w["lens"], 32, d, d)
     nbytes = gen.prefill_bytes(w["lens"], 32, 8, d, d)
     ms = wall / steps * 1e3
-    return dict(name=f"varlen causal batch prefill: 16 seqs L~U[128,8192] Hq32/Hk8 D{d} paged P=128 (bf16)",
+    tag = (" + ALiBi" if alibi else "") + (" [K/V cache fp8 e4m3]" if kv_fp8 else "") + (f" [tile variant {variant}]" if variant else "")
+    return dict(name=f"varlen causal batch prefill: 16 seqs L~U[128,8192] Hq32/Hk8 D{d} paged P=128 (bf16)" + tag,
                 ms_per_step=ms, flops=flops, bytes=nbytes, tflops=flops / (ms * 1e-3) / 1e12, kernel_ms=kern_ms,
                 kernel_tflops=flops / (kern_ms * 1e-3) / 1e12, total_q=sum(w["lens"]), kernel=kernel)
 
@@ -332,11 +341,22 @@ def main():
             r4 = bench_appendkv(args, torch, fmha, gen, 100, 10)
             return dict(workload=r4["name"], us_per_call=r4["us_per_call"], bytes=r4["bytes"], new_tokens=r4["new_tokens"])
 
-        def prefill(d):
-            r5 = bench_prefill(args, torch, fmha, gen, d, 10, 3)
+        def prefill(d, **kw):
+            r5 = bench_prefill(args, torch, fmha, gen, d, 10, 3, **kw)
             return dict(workload=r5["name"], ms_per_call=r5["ms_per_step"], tflops=r5["tflops"],
                         mfma_util_pct=100 * r5["tflops"] / MFMA_BF16_PEAK_TFLOPS, flops=r5["flops"], kernel_ms=r5["kernel_ms"],
                         kernel=r5["kernel"])
+
+        def prefill_tuned():
+            # every tile variant of the ping-pong kernel on this workload, then the fastest again as a line of its own
+            tried = {}
+            for v in (1, 2, 3, 4):
+                r = bench_prefill(args, torch, fmha, gen, 128, 5, 2, variant=v)
+                tried[f"v{v}"] = dict(ms=r["kernel_ms"], kernel=r["kernel"])
+            best = min((1, 2, 3, 4), key=lambda v: tried[f"v{v}"]["ms"])
+            out = prefill(128, variant=best)
+            out.update(variant=best, tried_kernel_ms={k: t["ms"] for k, t in tried.items()})
+            return out
 
         def splitkv_variant(path, ns, kv_fp8=False):
             a2 = argparse.Namespace(**vars(args))
@@ -355,6 +375,10 @@ def main():
         secondary("appendkv", append)
         for d in (128, 256):
             secondary(f"prefill_d{d}", lambda d=d: prefill(d))
+        secondary("prefill_d128_tuned", prefill_tuned)
+        secondary("prefill_d128_alibi", lambda: prefill(128, alibi=True))
+        secondary("prefill_d256_alibi", lambda: prefill(256, alibi=True))
+        secondary("prefill_d128_fp8_cache", lambda: prefill(128, kv_fp8=True))
 
     line = {
         "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -449,6 +449,7 @@ int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o
     a.hq = (int32_t)hq;
     a.dv = (int32_t)dv;
     a.num_splits = (int32_t)num_splits;
+    a.num_cu = cu_count();
     return launch_status(fck::launch_splitkv_combine(a, dtype, static_cast<hipStream_t>(stream)), "FmhaFwdSplitKVCombine launch");
 }
 

@@ -59,6 +59,7 @@ struct CombineArgs {
     int64_t rows;  // Bs * Sq
     int64_t Sq;
     int32_t hq, dv, num_splits;
+    int32_t num_cu;  // compute units of the device (decides the workgroup size)
 };
 
 struct AppendKvArgs {

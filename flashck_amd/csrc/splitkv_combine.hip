@@ -3,16 +3,19 @@
 // A pure streaming reduce: DV/4 lanes own one output row with float4 loads of each split's partial row.
 // Layouts: o_acc [Bs, Hq, ns, Sq, Dv], lse_acc [Bs, Hq, ns, Sq], o [Bs*Sq, Hq, Dv].  Dv is any multiple of 8 up to 256: the
 // kernel is instantiated for DV = 64 / 128 / 256 and the lanes past Dv of a row's group idle.
+// The work is a short chain of dependent loads per row, so what matters is how many CUs share it: workgroups are
+// 256 threads when that still gives every CU a few of them, one wave (64 threads) otherwise - a decode step of 256
+// output rows then runs on 128 workgroups instead of 32.
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace fck {
 
-template <typename T, int DV>
-__global__ __launch_bounds__(256) void splitkv_combine_kernel(const CombineArgs a)
+template <typename T, int DV, int NT = 256>
+__global__ __launch_bounds__(NT) void splitkv_combine_kernel(const CombineArgs a)
 {
     constexpr int TPR = DV / 4;     // threads per output row
-    constexpr int RPB = 256 / TPR;  // rows per block
+    constexpr int RPB = NT / TPR;   // rows per block
     const int64_t item = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;  // (row, head) pair
     const int c = (threadIdx.x % TPR) * 4;
     if (item >= a.rows * a.hq || c >= a.dv) return;
@@ -32,10 +35,14 @@ __global__ __launch_bounds__(256) void splitkv_combine_kernel(const CombineArgs 
 template <typename T, int DV>
 static hipError_t launch_dv(const CombineArgs& a, hipStream_t st)
 {
-    constexpr int RPB = 256 / (DV / 4);
+    constexpr int RPB = 256 / (DV / 4), RPW = 64 / (DV / 4);  // rows per 256-thread / per 64-thread workgroup
     const int64_t items = a.rows * a.hq;
-    const dim3 grid((unsigned)((items + RPB - 1) / RPB));
-    hipLaunchKernelGGL((splitkv_combine_kernel<T, DV>), grid, dim3(256), 0, st, a);
+    const int64_t wide = (items + RPB - 1) / RPB;
+    if (wide < 4 * (int64_t)a.num_cu) {
+        hipLaunchKernelGGL((splitkv_combine_kernel<T, DV, 64>), dim3((unsigned)((items + RPW - 1) / RPW)), dim3(64), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((splitkv_combine_kernel<T, DV, 256>), dim3((unsigned)wide), dim3(256), 0, st, a);
+    }
     return hipGetLastError();
 }
 

@@ -41,3 +41,17 @@ def test_group_mode_layout(fmha, orc):
     o = fmha.fmha_fwd_splitkv_combine(dev(lse), dev(o_acc), torch.bfloat16, cu_seqlens_q=dev(cu), max_seqlen_q=5)
     ref = orc.splitkv_combine(lse, o_acc, torch.bfloat16, seqstart_q=cu)
     assert_close(o, ref, 2e-2, "group combine")
+
+
+@pytest.mark.parametrize("dv,rows", [(64, 170), (128, 90), (256, 45)])
+def test_combine_many_rows(fmha, orc, dv, rows):
+    """Enough output rows that the launcher takes 256-thread workgroups (small problems run one wave per workgroup):
+    both workgroup shapes, incl. a last workgroup that is only partly filled."""
+    g = torch.Generator().manual_seed(dv + rows)
+    B, H, ns = 3, 33, 3
+    o_acc = torch.randn(B, H, ns, rows, dv, generator=g)
+    lse = torch.randn(B, H, ns, rows, generator=g) * 2
+    lse[2, 5, 1, :] = float("-inf")
+    o = fmha.fmha_fwd_splitkv_combine(dev(lse), dev(o_acc), torch.bfloat16)
+    ref = orc.splitkv_combine(lse, o_acc, torch.bfloat16)
+    assert_close(o, ref, 2e-2, "combine, many rows")
