@@ -72,7 +72,7 @@ def parse():
                     help="two-launch: split-KV + combine kernels with a caller-owned workspace; fused: one launch "
                          "(--num-splits 0 lets the library choose the key ranges)")
     args = ap.parse_args()
-    # the split-KV workload as BASELINE config 3 states it
+    # the split-KV workload: 32768 keys per sequence, 8 splits, shuffled pages
     args.kv_len, args.num_splits, args.no_shuffle = 32768, 8, False
     return args
 

@@ -1,5 +1,5 @@
 """GPU: the compiled `flash_ck` module (torch tensors in and out, as the reference's pybind layer) against the oracle:
-BASELINE config 1 by module name, then one small case per operator."""
+the dense fp16 benchmark workload (batch 2, 128 tokens, 8 heads, head dim 64) by module name, then one small case per operator."""
 import math
 
 import pytest
