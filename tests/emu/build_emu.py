@@ -33,9 +33,27 @@ def _compile(path):
     return obj
 
 
+class _Locked:
+    """one build at a time (test workers of a parallel run all ask for the library)"""
+
+    def __enter__(self):
+        import fcntl
+        os.makedirs(OBJ, exist_ok=True)
+        self.f = open(os.path.join(OBJ, ".lock"), "w")
+        fcntl.flock(self.f, fcntl.LOCK_EX)
+
+    def __exit__(self, *exc):
+        self.f.close()
+
+
 def build():
+    with _Locked():
+        return _build()
+
+
+def _build():
     os.makedirs(OBJ, exist_ok=True)
-    paths = [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(HERE, "emu_runtime.cpp")]
+    paths = [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(HERE, "emu_runtime.cpp"), os.path.join(HERE, "selftest.cpp")]
     with ThreadPoolExecutor(max_workers=min(len(paths), os.cpu_count() or 4)) as ex:
         objs = list(ex.map(_compile, paths))
     if os.path.exists(LIB) and os.path.getmtime(LIB) >= max(os.path.getmtime(o) for o in objs):
@@ -53,9 +71,10 @@ def build_pybind():
     from flash_ck import build as fb
     out = os.path.join(HERE, "flash_ck_emu" + sysconfig.get_config_var("EXT_SUFFIX"))
     src = os.path.join(ROOT, "flash_ck", "csrc", "pybind.cpp")
-    if os.path.exists(out) and os.path.getmtime(out) > max(os.path.getmtime(src), os.path.getmtime(LIB)):
-        return out
-    return fb.build(name="flash_ck_emu", out=out, kernel_lib=LIB, extra=["-DFLASH_CK_HOST_TENSORS"])
+    with _Locked():
+        if os.path.exists(out) and os.path.getmtime(out) > max(os.path.getmtime(src), os.path.getmtime(LIB)):
+            return out
+        return fb.build(name="flash_ck_emu", out=out, kernel_lib=LIB, extra=["-DFLASH_CK_HOST_TENSORS"])
 
 
 if __name__ == "__main__":

@@ -127,6 +127,7 @@ void fiber_exit()
 void fiber_main()
 {
     (*g.body)();
+    if (cur->pending_count) fail("a lane ended with global -> LDS copies still in flight (no wait before the workgroup retires)");
     fiber_exit();
 }
 
@@ -169,6 +170,38 @@ const char* exchange(const void* mine, size_t n)
         while (w.gen == gen && !g.failed) yield_waiting();
     }
     return &slots[0][0];
+}
+
+bool late_loads()
+{
+    static const bool late = [] {
+        const char* e = getenv("EMU_LATE_LOADS");
+        return !(e && e[0] == '0');
+    }();
+    return late;
+}
+
+void request_copy(char* dst, const char* src)
+{
+    if (!late_loads()) {
+        memcpy(dst, src, 16);
+        return;
+    }
+    Lane& l = *cur;
+    if (l.pending_count == 256) land_copies(255);  // more than the hardware counter holds: the oldest must have landed
+    l.pending[(l.pending_head + l.pending_count) & 255] = PendingCopy{dst, src};
+    ++l.pending_count;
+}
+
+void land_copies(int keep)
+{
+    Lane& l = *cur;
+    while (l.pending_count > keep) {
+        const PendingCopy& c = l.pending[l.pending_head];
+        memcpy(c.dst, c.src, 16);
+        l.pending_head = (l.pending_head + 1) & 255;
+        --l.pending_count;
+    }
 }
 
 int readfirstlane(int x) { return lane_value<int>(exchange(&x, 4), 0); }
@@ -221,6 +254,7 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
                     f.lane.gdim = grid;
                     f.lane.lane = t & 63;
                     f.lane.wave = t >> 6;
+                    f.lane.pending_head = f.lane.pending_count = 0;
                     f.done = false;
                     ++g.waves[t >> 6].live;
                     // initial frame: six callee-saved registers, then the entry point as return address; the stack

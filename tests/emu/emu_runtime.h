@@ -50,16 +50,34 @@ inline const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "n
 
 namespace emu {
 
+// A global -> LDS copy a lane has requested and that has not landed yet (see late_loads()).
+struct PendingCopy {
+    char* dst;
+    const char* src;
+};
+
 struct Lane {
     dim3 tid;  // threadIdx of the fiber that is running
     dim3 bid, bdim, gdim;
     int lane, wave;
+    PendingCopy pending[256];  // FIFO: vector-memory operations complete in order
+    int pending_head, pending_count;
 };
 extern thread_local Lane* cur;
 
 // last launch failed (a kernel broke a rule of the emulator: see emu_runtime.cpp); cleared by the read
 hipError_t take_error();
 void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>& body);
+// How the asynchronous global -> LDS copies are modelled.  true (default): a copy lands at the LAST moment the
+// program allows - when the lane that requested it waits for its outstanding copies to drop below the copy's place in
+// the queue, or when the lane ends - so a read that is not covered by the proper wait sees stale (poisoned) LDS and the
+// parity test fails.  false (EMU_LATE_LOADS=0): copies land at once, the earliest moment, which is what exposes a
+// request into a buffer that is still being read.
+bool late_loads();
+// the lane's part of one global -> LDS instruction: 16 bytes from src to dst
+void request_copy(char* dst, const char* src);
+// leave at most `keep` of the lane's copies outstanding (the oldest land first)
+void land_copies(int keep);
 char* dynamic_lds();
 void barrier();
 // Rendezvous of the wave: deposits n <= 256 bytes, returns when every live lane of the wave has deposited; the

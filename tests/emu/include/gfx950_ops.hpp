@@ -33,16 +33,18 @@ inline void swap16(float x, float& a, float& b)
     b = emu::lane_value<float>(all, l | 16);
 }
 
-// global -> LDS: lane l copies 16 bytes to byte l * 16 of the 1 KiB block at dst (at once: nothing is asynchronous here)
+// global -> LDS: lane l copies 16 bytes to byte l * 16 of the 1 KiB block at dst; when the copy lands: emu::late_loads()
 inline void load_to_lds(uint32_t dst, const void* base, uint32_t off)
 {
-    memcpy((char*)(uintptr_t)dst + emu::cur->lane * 16, (const char*)base + off, 16);
+    emu::request_copy((char*)(uintptr_t)dst + emu::cur->lane * 16, (const char*)base + off);
 }
-inline void load_to_lds(uint32_t dst, const void* src) { memcpy((char*)(uintptr_t)dst + emu::cur->lane * 16, src, 16); }
+inline void load_to_lds(uint32_t dst, const void* src) { emu::request_copy((char*)(uintptr_t)dst + emu::cur->lane * 16, (const char*)src); }
 
+// the kernels count only their own global -> LDS instructions; so does this
 template <int N>
 inline void wait_vm()
 {
+    emu::land_copies(N);
 }
 
 #define FCK_ACC_SCALE(acc, f) ((acc) *= (f))

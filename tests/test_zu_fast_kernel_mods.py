@@ -80,3 +80,20 @@ def test_narrow_bias_is_clamped_to_its_last_column(fmha, orc, path):
     ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqlen_k=kv["seqlen_k"], block_table=kv["block_table"],
                       mask_type=0 if path == "decode" else 2, window=(-1, -1) if path == "decode" else (-1, 0), bias=wide)
     assert_close(o, ro, 2e-2, f"narrow bias, {path}")
+
+
+@pytest.mark.parametrize("d,page,sk", [(64, 64, 4400), (128, 128, 8300), (256, 64, 4200)])
+@pytest.mark.parametrize("mask", [(2, (-1, 0)), (0, (-1, -1)), (2, (300, 0))])
+def test_few_query_rows_over_many_key_tiles(fmha, orc, d, page, sk, mask):
+    """200 query rows over up to 130 key tiles of one sequence: the ring buffers wrap many times and the per-workgroup
+    cache of first rows is reloaded (it holds 64 tiles per register), at the cost of a short test."""
+    g = torch.Generator().manual_seed(d + sk)
+    dtype, hq, hk, sq = torch.bfloat16, 2, 1, 200
+    kv = gen.paged_kv([sk, 130], hk, d, dtype, g, page)
+    q = gen.randn((2, sq, hq, d), dtype, g)
+    o = fmha.fmha_fwd_pagedkv(dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]), dev(kv["seqlen_k"]), dev(kv["block_table"]), mask_type=mask[0],
+                              window=mask[1])
+    name = _lib.load().fck_fmha_last_kernel()
+    assert name == (b"prefill_dma_kernel<uniform_page>" if d == 256 else b"prefill_pp_kernel<uniform_page>")
+    ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], mask_type=mask[0], window=mask[1])
+    assert_close(o, ro, 2e-2, f"{name.decode()}, {sk} keys")
