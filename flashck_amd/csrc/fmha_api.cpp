@@ -256,9 +256,9 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
     if (attrs && attrs->decode_variant != 0) {
         if (attrs->decode_variant != 1 && attrs->decode_variant != 2)
             return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant %d out of range [0,2]", attrs->decode_variant);
-        if (attrs->decode_variant == 2 && (hk % 2 || d > 128 || padded || q_max_seq_len * (hq / hk) > 16 || a.mod.active()))
-            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant 2 (head pairs) needs an even kv_num_heads, head dim 64 or 128, at most 16 "
-                                                  "packed query rows and no bias / soft cap");
+        if (attrs->decode_variant == 2 && (hk % 2 || d > 128 || padded || q_max_seq_len * (hq / hk) > 16))
+            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant 2 (head pairs) needs an even kv_num_heads, head dim 64 or 128 and at most 16 "
+                                                  "packed query rows");
         a.variant = attrs->decode_variant;
     }
     if (attrs && attrs->kv_dtype != 0) {

@@ -67,7 +67,6 @@ __device__ __forceinline__ int v_swizzle(int key)
 template <typename T, int D, int NW, int MB, int HG, bool kUniformPage, bool kMod = false, bool kKv8 = false, bool kPad = false>
 __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvArgs a)
 {
-    static_assert(!kMod || HG == 1, "score modifiers are per head: one KV head per workgroup");
     static_assert(!kPad || (HG == 1 && !kKv8), "padded head dims: one KV head per workgroup, 16-bit cache");
     const int dq = kPad ? a.d : D;   // elements per stored Q / K row
     const int dvs = kPad ? a.dv : D;  // elements per stored V / partial-output row
@@ -158,12 +157,14 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
         }
     }
     // bias / ALiBi / soft cap of this lane's rows
-    RowMod<T> rmod[MB];
+    RowMod<T> rmod[HG][MB];  // per head of the group: slopes and bias rows differ between heads
     if constexpr (kMod) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-            rmod[mb].init(a.mod, b, q_row0, hkv0 * g + row_hl[mb], row_i[mb], sq_b, sk_b, a.mask_type, a.window_left, a.window_right,
-                          a.seqstart_q != nullptr);
+        for (int hl = 0; hl < HG; ++hl)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                rmod[hl][mb].init(a.mod, b, q_row0, (hkv0 + hl) * g + row_hl[mb], row_i[mb], sq_b, sk_b, a.mask_type, a.window_left,
+                                  a.window_right, a.seqstart_q != nullptr);
     }
     // key range any row of the tile can see (uniform)
     const int i_first = r_tile0 / g;
@@ -382,7 +383,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
                         const bool vis = key >= lo[mb] && key < hi[mb];
                         float v;
                         if constexpr (kMod)
-                            v = vis ? rmod[mb].score(s[mb][nb][j], key) : -INFINITY;
+                            v = vis ? rmod[hl][mb].score(s[mb][nb][j], key) : -INFINITY;
                         else
                             v = vis ? s[mb][nb][j] * a.scale_log2 : -INFINITY;
                         x[nb * 4 + j] = v;
@@ -590,14 +591,14 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
             if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true, false, true>>(grid, block, lds, st, a);
             return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true, false, true>>(grid, block, lds, st, a);
         }
-        if (a.mod.active()) {
-            if (a.kv8) {
-                if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true, true>>(grid, block, lds, st, a);
-                return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true, true>>(grid, block, lds, st, a);
-            }
-            if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true>>(grid, block, lds, st, a);
-            return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true>>(grid, block, lds, st, a);
+    }
+    if (a.mod.active()) {
+        if (a.kv8) {
+            if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true, true>>(grid, block, lds, st, a);
+            return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true, true>>(grid, block, lds, st, a);
         }
+        if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true>>(grid, block, lds, st, a);
+        return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true>>(grid, block, lds, st, a);
     }
     if (a.kv8) {
         if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, false, true>>(grid, block, lds, st, a);
@@ -612,7 +613,7 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
 static bool use_head_pairs(const SplitKvArgs& a, int m_tiles, int num_cu)
 {
     if (a.variant != 0) return a.variant == 2;  // validated by the caller
-    if (a.hk % 2 || a.mod.active() || a.d != a.dv || (a.d != 64 && a.d != 128)) return false;
+    if (a.hk % 2 || a.d != a.dv || (a.d != 64 && a.d != 128)) return false;
     return (int64_t)(a.hk / 2) * a.num_splits * m_tiles * a.batch >= num_cu;
 }
 

@@ -662,8 +662,9 @@ def _usable_variant(variant, q_num_heads, kv_num_heads, rows, head_dim, v_head_d
     """A kernel variant from the tuning cache is a hint: the record's problem class is coarser than what the variant
     needs (query counts are bucketed, v_head_dim is not part of the key), so its preconditions are checked again for
     this call, and 0 (the library's choice) is returned when one fails.  Head pairs (2) need an even number of KV heads,
-    equal head dims of 64 or 128, at most 16 packed query rows (queries x heads per KV head) and no score modifier /
-    fp8 cache; one head per workgroup (1) fits every call."""
+    equal head dims of 64 or 128 and at most 16 packed query rows (queries x heads per KV head); a record is only served to
+    the kind of call it was measured with (plain: no score modifier, 16-bit cache); one head per workgroup (1) fits
+    every call."""
     variant = int(variant)
     if variant == 2:
         g = q_num_heads // max(kv_num_heads, 1)

@@ -93,7 +93,7 @@ typedef struct fck_fmha_attrs {
     /* Split-KV kernel variant, the counterpart of the tile instance FlashCK's tuner picks per problem
      * (core/profiling/profiling_db.cc:64-71): 0 = the library chooses; 1 = one KV head per workgroup (32-key tiles);
      * 2 = two adjacent KV heads per workgroup (16-key tiles, 512-byte row pieces; needs an even kv_num_heads, at most
-     * 16 packed query rows, head dim <= 128 and no bias / soft cap).  A variant the problem cannot take is an error. */
+     * 16 packed query rows and head dim 64 or 128).  A variant the problem cannot take is an error. */
     int32_t decode_variant;
     /* Prefill tile variant, likewise: 0 = the library chooses; 1 = the default schedule of the kernel the call takes;
      * 2..4 = variants of the 8-wave ping-pong kernel (2: byte offsets of whole-tile requests computed once per

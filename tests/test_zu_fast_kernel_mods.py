@@ -97,3 +97,32 @@ def test_few_query_rows_over_many_key_tiles(fmha, orc, d, page, sk, mask):
     assert name == (b"prefill_dma_kernel<uniform_page>" if d == 256 else b"prefill_pp_kernel<uniform_page>")
     ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], mask_type=mask[0], window=mask[1])
     assert_close(o, ro, 2e-2, f"{name.decode()}, {sk} keys")
+
+
+@pytest.mark.parametrize("kind", ["cap", "alibi_h", "alibi_b", "alibi_cap", "bias"])
+@pytest.mark.parametrize("d,page,fp8", [(128, 128, False), (64, 64, False), (128, 48, False), (128, 128, True)])
+def test_head_pair_decode_with_score_modifiers(fmha, orc, kind, d, page, fp8):
+    """Score modifiers on the split-KV variant that streams two KV heads per workgroup (forced through the attribute;
+    the two heads of a pair have different slopes and bias rows); also over an fp8 cache."""
+    g = torch.Generator().manual_seed(3 + d + page)
+    dtype, hq, hk, B = torch.bfloat16, 16, 4, 5
+    lens = [1, 17, 129, 700, 333]
+    kv = gen.paged_kv(lens, hk, d, dtype, g, page)
+    q = gen.randn((B, 2, hq, d), dtype, g)        # 2 queries x 4 heads per KV head = 8 packed rows
+    if kind == "bias":
+        kw = dict(bias=gen.randn((B, hq, 2, 704), dtype, g))
+    else:
+        kw = _mods(kind, hq, B, g)
+    kc, vc, skw = kv["k_cache"], kv["v_cache"], {}
+    if fp8:
+        skw = dict(k_descale=0.03, v_descale=0.04)
+        kc, vc = (kc.float() / 0.03).to(torch.float8_e4m3fn), (vc.float() / 0.04).to(torch.float8_e4m3fn)
+    common = dict(seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], scale=1 / math.sqrt(d), mask_type=2, window=(-1, 0))
+    o_acc, lse_acc = fmha.fmha_fwd_splitkv(dev(q), dev(kc), dev(vc), 3, decode_variant=2, **{k: dev(v) for k, v in {**common, **kw}.items()}, **skw)
+    name = _lib.load().fck_fmha_last_kernel()
+    assert b"head_pairs" in name and b"score_mod" in name and (b"kv_fp8" in name) == fp8
+    o = fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype)
+    ro = orc.fmha_fwd(q, kc, vc, **common, **kw, **skw)
+    assert_close(o, ro, 2e-2, f"{kind} on {name.decode()}")
+    o1, l1 = fmha.fmha_fwd_splitkv(dev(q), dev(kc), dev(vc), 3, decode_variant=1, **{k: dev(v) for k, v in {**common, **kw}.items()}, **skw)
+    assert_close(fmha.fmha_fwd_splitkv_combine(l1, o1, dtype), ro, 2e-2, f"{kind}, one head per workgroup")
