@@ -163,7 +163,7 @@ def bench_decode(args, torch, fmha, gen, which):
             fmha.fmha_fwd_splitkv_fused(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], out=o)
         else:
             fmha.fmha_fwd_splitkv(q, kc, vc, ns, seqlen_k=sl, block_table=bt, scale=w["scale"], o_acc=o_acc, lse_acc=lse_acc,
-                                  decode_variant=variant, **scales)
+                                  decode_variant=variant, max_seqlen_k=max(w["lens"]) if variant >= 3 else 0, **scales)
         if ev is not None:
             ev[1].record()
         if not fused:
@@ -327,7 +327,7 @@ def main():
             w = gen.workload_paged_decode()
             t = [w[k].to("cuda") for k in ("q", "k_cache", "v_cache", "seqlen_k", "block_table")]
             with tempfile.TemporaryDirectory() as tmp:
-                rec = fmha.tune_decode_num_splits(*t, max_seqlen_k=max(w["lens"]), candidates=(1, 2, 3, 4, 6, 8), variants=(1, 2),
+                rec = fmha.tune_decode_num_splits(*t, max_seqlen_k=max(w["lens"]), candidates=(1, 2, 3, 4, 6, 8, 12, 16), variants=(1, 2, 3, 4),
                                                   cache=tuning.TuningCache(directory=tmp), scale=w["scale"])
             del t
             a2 = argparse.Namespace(**vars(args))

@@ -18,14 +18,14 @@ namespace {
 thread_local char g_err[512] = "";
 thread_local const char* g_kernel = "";  // kernel family of the calling thread's last launch
 
-// "splitkv_decode_kernel<uniform_page|row_lookup[,head_pairs][,kv_fp8][,score_mod][,padded_head_dim][,fused]>": the
+// "splitkv_decode_kernel<uniform_page|row_lookup[,head_pairs][,kv_fp8][,score_mod][,padded_head_dim][,fused][,equal_chunks]>": the
 // variant the calling thread's last split-KV launch took
-void name_decode_kernel(bool uniform, int heads_per_workgroup, bool kv8, bool mod, bool padded, bool fused)
+void name_decode_kernel(bool uniform, int heads_per_workgroup, bool kv8, bool mod, bool padded, bool fused, bool chunks)
 {
     thread_local char name[128];
-    snprintf(name, sizeof(name), "splitkv_decode_kernel<%s%s%s%s%s%s>", uniform ? "uniform_page" : "row_lookup",
+    snprintf(name, sizeof(name), "splitkv_decode_kernel<%s%s%s%s%s%s%s>", uniform ? "uniform_page" : "row_lookup",
              heads_per_workgroup == 2 ? ",head_pairs" : "", kv8 ? ",kv_fp8" : "", mod && !padded ? ",score_mod" : "",
-             padded ? ",padded_head_dim" : "", fused ? ",fused" : "");
+             padded ? ",padded_head_dim" : "", fused ? ",fused" : "", chunks ? ",equal_chunks" : "");
     g_kernel = name;
 }
 
@@ -254,12 +254,25 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
     if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
     a.v_descale = 1.f;
     if (attrs && attrs->decode_variant != 0) {
-        if (attrs->decode_variant != 1 && attrs->decode_variant != 2)
-            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant %d out of range [0,2]", attrs->decode_variant);
-        if (attrs->decode_variant == 2 && (hk % 2 || d > 128 || padded || q_max_seq_len * (hq / hk) > 16))
-            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant 2 (head pairs) needs an even kv_num_heads, head dim 64 or 128 and at most 16 "
-                                                  "packed query rows");
-        a.variant = attrs->decode_variant;
+        const int32_t dvar = attrs->decode_variant;
+        if (dvar < 1 || dvar > 4) return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant %d out of range [0,4]", dvar);
+        if ((dvar == 2 || dvar == 4) && (hk % 2 || d > 128 || padded || q_max_seq_len * (hq / hk) > 16))
+            return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant %d (head pairs) needs an even kv_num_heads, head dim 64 or 128 and at most 16 "
+                                                  "packed query rows", dvar);
+        if (dvar >= 3) {
+            // splits of equal size in keys: a plain call over a block table with tile-aligned pages, one 16-row block
+            if (!block_table || page_block_size % 32 || d > 128 || padded || q_max_seq_len * (hq / hk) > 16 || a.mod.active() || attrs->kv_dtype != 0)
+                return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant %d (splits of equal size) needs a block table with pages a multiple of 32 keys, head "
+                                                      "dim 64 or 128, at most 16 packed query rows and no bias / soft cap / fp8 cache", dvar);
+            if (attrs->max_seqlen_k < 0) return fail(FCK_ERR_INVALID_ARGUMENT, "max_seqlen_k must be >= 0 (0: the block table's capacity)");
+            const int64_t capacity = (batch > 0 ? max_num_page_blocks / batch : 0) * page_block_size;
+            const int64_t bound = attrs->max_seqlen_k > 0 && attrs->max_seqlen_k < capacity ? attrs->max_seqlen_k : capacity;
+            int64_t chunk = (bound + num_splits - 1) / num_splits;
+            chunk = (chunk + 31) / 32 * 32;
+            if (chunk <= 0 || chunk > INT32_MAX) return fail(FCK_ERR_INVALID_ARGUMENT, "decode_variant %d: no positive key-count bound", dvar);
+            a.split_chunk = (int32_t)chunk;
+        }
+        a.variant = dvar;
     }
     if (attrs && attrs->kv_dtype != 0) {
         // fp8 K/V with static per-tensor scales: the K scale multiplies every score, the V scale the output
@@ -337,7 +350,7 @@ int fck_fmha_fwd_splitkv_attrs(const void* q, const void* k, const void* v, cons
     a.lse_acc = static_cast<float*>(lse_acc);
     int hpw = 1;
     const hipError_t e = fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream), &hpw);
-    name_decode_kernel(uniform, hpw, a.kv8 != 0, a.mod.active(), d != dv || d != kernel_dim(d, dv), false);
+    name_decode_kernel(uniform, hpw, a.kv8 != 0, a.mod.active(), d != dv || d != kernel_dim(d, dv), false, a.split_chunk > 0);
     return launch_status(e, "FmhaFwdSplitKV launch");
 }
 
@@ -386,7 +399,7 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
     a.o = o;
     int hpw = 1;
     const hipError_t e = fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream), &hpw);
-    name_decode_kernel(uniform, hpw, false, false, false, true);
+    name_decode_kernel(uniform, hpw, false, false, false, true, false);
     return launch_status(e, "FmhaFwdSplitKV (fused) launch");
 }
 

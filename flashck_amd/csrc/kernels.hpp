@@ -45,7 +45,8 @@ struct SplitKvArgs {
     uint32_t mask_type;
     int64_t window_left, window_right;
     ScoreMod mod;      // bias / ALiBi / soft cap; all zero: none
-    int32_t variant;   // 0: chosen by the launcher; 1: one KV head per workgroup; 2: head pairs
+    int32_t variant;   // 0: chosen by the launcher; 1 / 3: one KV head per workgroup; 2 / 4: head pairs (3, 4: with split_chunk)
+    int32_t split_chunk;  // > 0: keys per split, the same for every sequence (variants 3 and 4); 0: num_splits equal parts per sequence
     int32_t kv8;       // K and V are fp8 (e4m3); the K scale is folded into scale_log2 / mod.scale by the caller
     float v_descale;   // factor on the output (1 unless V is quantised)
     int32_t longest_first;  // set by the launcher: workgroups take the sequences in order of decreasing key count

@@ -64,7 +64,12 @@ __device__ __forceinline__ int v_swizzle(int key)
 // kPad: the stored head dims (a.d for Q/K, a.dv for V and the output; multiples of 8) are smaller than D: rows are
 // a.d / a.dv elements apart, and the 16-byte pieces past a row's end are zeros instead of loads (a zero column of Q and K
 // adds nothing to a score, a zero column of V gives an output column that is not stored).
-template <typename T, int D, int NW, int MB, int HG, bool kUniformPage, bool kMod = false, bool kKv8 = false, bool kPad = false>
+// kChunk: the key ranges of the splits are chunks of a.split_chunk keys, the same for every sequence (split s of a
+// sequence covers [s * chunk, (s + 1) * chunk), the last split also whatever lies beyond), instead of num_splits equal
+// parts of each sequence: work items of equal size for a ragged batch; the splits a short sequence does not reach are
+// empty.
+template <typename T, int D, int NW, int MB, int HG, bool kUniformPage, bool kMod = false, bool kKv8 = false, bool kPad = false,
+          bool kChunk = false>
 __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvArgs a)
 {
     static_assert(!kPad || (HG == 1 && !kKv8), "padded head dims: one KV head per workgroup, 16-bit cache");
@@ -132,10 +137,10 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
     if (r_tile0 >= R) return;
 
     // Split geometry: num_splits equal ranges of ceil(sk / num_splits) keys (the last ones may be empty)
-    const int per = max(1, (sk_b + a.num_splits - 1) / a.num_splits);
+    const int per = kChunk ? a.split_chunk : max(1, (sk_b + a.num_splits - 1) / a.num_splits);
     const int n_active = a.num_splits;
     const int k0 = (int)min((int64_t)per * split, (int64_t)sk_b);
-    const int k1 = min(k0 + per, sk_b);
+    const int k1 = (kChunk && split == a.num_splits - 1) ? sk_b : min(k0 + per, sk_b);
 
     const MaskYX mk = make_mask(a.mask_type, a.window_left, a.window_right, sq_b, sk_b);
 
@@ -604,6 +609,14 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
         if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, false, true>>(grid, block, lds, st, a);
         return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, false, true>>(grid, block, lds, st, a);
     }
+    if (a.split_chunk > 0) {  // validated by the caller: plain call, uniform pages, one 16-row block, head dim 64 or 128
+        if constexpr (NW == 8 && MB == 1 && D <= 128) {
+            if (!uniform || a.tickets) return hipErrorInvalidValue;
+            return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, false, false, false, true>>(grid, block, lds, st, a);
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
     if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true>>(grid, block, lds, st, a);
     return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false>>(grid, block, lds, st, a);
 }
@@ -612,7 +625,7 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
 // covers the CUs.
 static bool use_head_pairs(const SplitKvArgs& a, int m_tiles, int num_cu)
 {
-    if (a.variant != 0) return a.variant == 2;  // validated by the caller
+    if (a.variant != 0) return a.variant == 2 || a.variant == 4;  // validated by the caller
     if (a.hk % 2 || a.d != a.dv || (a.d != 64 && a.d != 128)) return false;
     return (int64_t)(a.hk / 2) * a.num_splits * m_tiles * a.batch >= num_cu;
 }

@@ -123,7 +123,7 @@ def _window(window):
 
 
 def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols, kv_fp8=False, k_descale=1.0, v_descale=1.0,
-           decode_variant=0, prefill_variant=0):
+           decode_variant=0, prefill_variant=0, max_seqlen_k=0):
     """fck_fmha_attrs for a call, or None when no score modifier is asked for.
 
     bias (elementwise, BiasEnum ELEMENTWISE_BIAS): q's dtype, last dim contiguous; batch mode [1|B, 1|Hq, sq, >= sk],
@@ -133,8 +133,9 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
     cap = float(logits_soft_cap)
     if not (cap >= 0.0) or math.isinf(cap):
         raise ValueError("logits_soft_cap must be finite and >= 0")
-    if int(decode_variant) not in (0, 1, 2):
-        raise ValueError("decode_variant must be 0 (library's choice), 1 (one KV head per workgroup) or 2 (head pairs)")
+    if int(decode_variant) not in (0, 1, 2, 3, 4):
+        raise ValueError("decode_variant must be 0 (library's choice), 1 (one KV head per workgroup), 2 (head pairs), or 3 / 4 (the same "
+                         "with splits of equal size in keys)")
     if int(prefill_variant) not in (0, 1, 2, 3, 4):
         raise ValueError("prefill_variant must be 0 (library's choice) or 1..4 (see fck_fmha_attrs.prefill_variant)")
     if bias is None and alibi_slopes is None and cap == 0.0 and not kv_fp8 and not decode_variant and not prefill_variant:
@@ -145,6 +146,7 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
     a.size = ctypes.sizeof(_lib.Attrs)
     a.logits_soft_cap = cap
     a.decode_variant = int(decode_variant)
+    a.max_seqlen_k = max(int(max_seqlen_k), 0)
     a.prefill_variant = int(prefill_variant)
     if kv_fp8:
         if not (float(k_descale) > 0.0 and float(v_descale) > 0.0 and math.isfinite(k_descale) and math.isfinite(v_descale)):
@@ -307,10 +309,13 @@ def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scal
 def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=None, cache_batch_idx=None,
                      cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q: int = 0, scale: float = 0.0,
                      mask_type: int = MASK_NONE, window=(-1, -1), o_acc=None, lse_acc=None, bias=None, alibi_slopes=None,
-                     logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0, decode_variant: int = 0):
+                     logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0, decode_variant: int = 0,
+                     max_seqlen_k: int = 0):
     """Split-KV forward: returns the per-split partials (o_acc, lse_acc), to be merged by fmha_fwd_splitkv_combine.
     decode_variant: 0 = the library picks the kernel variant, 1 / 2 force it (what the tuner records, see
-    tune_decode_num_splits).
+    tune_decode_num_splits); 3 / 4 = 1 / 2 with splits of equal size in keys (chunks of ceil(max_seqlen_k / num_splits)
+    keys, the same for every sequence: even work items for a ragged batch; max_seqlen_k = 0 takes the block table's
+    capacity).
     bias / alibi_slopes / logits_soft_cap: see _attrs.  k and v may be torch.float8_e4m3fn (a quantised cache with the
     static per-tensor scales k_descale, v_descale: value = descale * stored); q and the output keep q's dtype.
 
@@ -360,7 +365,7 @@ def fmha_fwd_splitkv(q, k, v, num_splits: int, *, seqlen_k=None, block_table=Non
         _check_shape("lse_acc", lse_acc, (bs, Hq, int(num_splits), sq), q)
     wl, wr = _window(window)
     at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, sq, 1 if (group or block_table is not None) else sk,
-                      kv_fp8, k_descale, v_descale, decode_variant)
+                      kv_fp8, k_descale, v_descale, decode_variant, max_seqlen_k=max_seqlen_k)
     if at is None:
         _call("fck_fmha_fwd_splitkv", _ptr(q), _ptr(k), _ptr(v), None, _ptr(lse_acc), _ptr(o_acc), _ptr(cu_seqlens_q),
               _ptr(cu_seqlens_k), _ptr(seqlen_k), _ptr(block_table), _ptr(cache_batch_idx), B, sq, sk, Hq, Hk, D, Dv,
@@ -658,19 +663,21 @@ def _auto_num_splits(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, h
         "fp16" if dtype == torch.float16 else "bf16")
 
 
-def _usable_variant(variant, q_num_heads, kv_num_heads, rows, head_dim, v_head_dim, plain=True):
+def _usable_variant(variant, q_num_heads, kv_num_heads, rows, head_dim, v_head_dim, plain=True, page_size=128):
     """A kernel variant from the tuning cache is a hint: the record's problem class is coarser than what the variant
     needs (query counts are bucketed, v_head_dim is not part of the key), so its preconditions are checked again for
     this call, and 0 (the library's choice) is returned when one fails.  Head pairs (2) need an even number of KV heads,
     equal head dims of 64 or 128 and at most 16 packed query rows (queries x heads per KV head); a record is only served to
     the kind of call it was measured with (plain: no score modifier, 16-bit cache); one head per workgroup (1) fits
-    every call."""
+    every call.  Variants 3 / 4 (splits of equal size) are 1 / 2 for plain calls with at most 16 packed rows, head dim 64
+    or 128 and pages a multiple of 32 keys."""
     variant = int(variant)
-    if variant == 2:
-        g = q_num_heads // max(kv_num_heads, 1)
-        ok = (plain and kv_num_heads % 2 == 0 and head_dim == v_head_dim and head_dim in (64, 128)
-              and rows * g <= 16)
-        return 2 if ok else 0
+    g = q_num_heads // max(kv_num_heads, 1)
+    small = plain and head_dim == v_head_dim and head_dim in (64, 128) and rows * g <= 16
+    if variant in (2, 4):
+        return variant if small and kv_num_heads % 2 == 0 and (variant == 2 or page_size % 32 == 0) else 0
+    if variant == 3:
+        return 3 if small and page_size % 32 == 0 else 0
     return variant if variant == 1 else 0
 
 
@@ -707,7 +714,7 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
             max_seqlen_k = block_table.shape[1] * k_cache.shape[1]
         num_splits, cached_variant = _auto_num_splits(B, Hq, Hk, sq, max_seqlen_k, D, k_cache.shape[1], q.dtype)
         if not decode_variant:
-            decode_variant = _usable_variant(cached_variant, Hq, Hk, sq, D, v_cache.shape[3], plain)
+            decode_variant = _usable_variant(cached_variant, Hq, Hk, sq, D, v_cache.shape[3], plain, k_cache.shape[1])
     if fused:
         if not plain or decode_variant:
             raise NotImplementedError("the fused launch takes no bias / soft cap / fp8 cache / kernel variant")
@@ -719,7 +726,7 @@ def fmha_decode_paged(q, k_cache, v_cache, seqlen_k, block_table, *, num_splits:
                                       cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, scale=scale,
                                       mask_type=mask_type, window=window, o_acc=o_acc, lse_acc=lse_acc, bias=bias,
                                       alibi_slopes=alibi_slopes, logits_soft_cap=logits_soft_cap, k_descale=k_descale,
-                                      v_descale=v_descale, decode_variant=decode_variant)
+                                      v_descale=v_descale, decode_variant=decode_variant, max_seqlen_k=max_seqlen_k)
     return fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_q, max_seqlen_q=max_seqlen_q, out=out)
 
 
@@ -831,7 +838,7 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
         if max_seqlen_k <= 0:
             max_seqlen_k = block_table.shape[1] * page  # what the block table can address
         num_splits, decode_variant = _auto_num_splits(B, Hq, Hk, n, max_seqlen_k, D, page, q.dtype)
-        decode_variant = _usable_variant(decode_variant, Hq, Hk, n, D, Dv, plain=not kv_fp8)
+        decode_variant = _usable_variant(decode_variant, Hq, Hk, n, D, Dv, plain=not kv_fp8, page_size=page)
     else:
         decode_variant = 0
     # a lone new token sees every key: no mask needed unless a sliding window is asked for
@@ -844,7 +851,7 @@ def fmha_decode_step(q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, 
     fmha_fwd_splitkv(q, k_cache, v_cache, num_splits, seqlen_k=seqlen_new, block_table=block_table,
                      cu_seqlens_q=cu_seqlens_knew, max_seqlen_q=n if packed else 0, scale=scale, mask_type=mask_type,
                      window=window, o_acc=o_acc, lse_acc=lse_acc, decode_variant=decode_variant, k_descale=k_descale,
-                     v_descale=v_descale)
+                     v_descale=v_descale, max_seqlen_k=max_seqlen_k)
     o = fmha_fwd_splitkv_combine(lse_acc, o_acc, q.dtype, cu_seqlens_q=cu_seqlens_knew, max_seqlen_q=n if packed else 0,
                                  out=out)
     return o, seqlen_new

@@ -135,7 +135,7 @@ def choose_splitkv(heuristic: Callable[[], int], batch, q_num_heads, kv_num_head
             SPLITKV, splitkv_problem(batch, q_num_heads, kv_num_heads, seqlen_q, max_seqlen_k, head_dim, page_size, dtype))
         if rec is not None and 1 <= int(rec.get("num_splits", 0)) <= 128:
             variant = int(rec.get("variant", 0))
-            return int(rec["num_splits"]), (variant if variant in (0, 1, 2) else 0)
+            return int(rec["num_splits"]), (variant if variant in (0, 1, 2, 3, 4) else 0)
     return int(heuristic()), 0
 
 

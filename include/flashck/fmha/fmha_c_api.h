@@ -93,7 +93,13 @@ typedef struct fck_fmha_attrs {
     /* Split-KV kernel variant, the counterpart of the tile instance FlashCK's tuner picks per problem
      * (core/profiling/profiling_db.cc:64-71): 0 = the library chooses; 1 = one KV head per workgroup (32-key tiles);
      * 2 = two adjacent KV heads per workgroup (16-key tiles, 512-byte row pieces; needs an even kv_num_heads, at most
-     * 16 packed query rows and head dim 64 or 128).  A variant the problem cannot take is an error. */
+     * 16 packed query rows and head dim 64 or 128); 3 / 4 = as 1 / 2 with splits of equal size in keys instead of
+     * num_splits equal parts of every sequence: split s of a sequence covers keys [s * chunk, (s + 1) * chunk) with
+     * chunk = ceil(bound / num_splits) rounded up to 32, bound = max_seqlen_k below (the last split also takes whatever
+     * lies beyond), so the work items of a ragged batch have one size and the splits a short sequence does not reach
+     * are empty (lse_acc = -inf); the combine is unchanged.  3 / 4 need a block table with pages a multiple of 32 keys,
+     * at most 16 packed query rows, head dim 64 or 128 and no bias / soft cap / fp8 cache.  A variant the problem
+     * cannot take is an error. */
     int32_t decode_variant;
     /* Prefill tile variant, likewise: 0 = the library chooses; 1 = the default schedule of the kernel the call takes;
      * 2..4 = variants of the 8-wave ping-pong kernel (2: byte offsets of whole-tile requests computed once per
@@ -106,6 +112,9 @@ typedef struct fck_fmha_attrs {
      * so a bias narrower than a sequence's key count is never read out of bounds (the scores of such keys then use
      * the last column).  0: not stated, only the sequence's own key count bounds the reads. */
     int64_t bias_cols;
+    /* decode_variant 3 / 4: upper bound of the key counts of the batch (0 or anything above the block table's capacity:
+     * that capacity).  A bound below a real key count costs balance, not correctness. */
+    int64_t max_seqlen_k;
 } fck_fmha_attrs;
 
 #define FCK_OK 0

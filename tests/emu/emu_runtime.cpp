@@ -32,7 +32,8 @@ struct Group {
     std::vector<Fiber> fibers;
     std::vector<WaveState> waves;
     char* stacks = nullptr;
-    char* lds = nullptr;
+    char* lds_region = nullptr;  // kLdsBytes, then one inaccessible page
+    char* lds = nullptr;         // the launch's dynamic LDS: ends where the inaccessible page begins
     int n = 0, live = 0, running = -1;
     int bar_arrived = 0;
     unsigned bar_gen = 0;
@@ -225,12 +226,14 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
     }
     if (!g.stacks) {
         g.stacks = (char*)mmap(nullptr, kStack * kMaxThreads, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
-        g.lds = (char*)mmap(nullptr, kLdsBytes, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_32BIT, -1, 0);
-        if (g.stacks == MAP_FAILED || g.lds == MAP_FAILED) {
+        g.lds_region = (char*)mmap(nullptr, kLdsBytes + 4096, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_32BIT, -1, 0);
+        if (g.stacks == MAP_FAILED || g.lds_region == MAP_FAILED || mprotect(g.lds_region + kLdsBytes, 4096, PROT_NONE) != 0) {
             fprintf(stderr, "emu: cannot map fiber stacks / LDS\n");
             abort();
         }
     }
+    // an access past the end of the launch's LDS allocation runs into the inaccessible page
+    g.lds = g.lds_region + kLdsBytes - ((lds_bytes + 15) & ~(size_t)15);
     g.fibers.resize(n);
     g.waves.resize((n + 63) / 64);
     g.n = n;
@@ -240,7 +243,7 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
         for (unsigned by = 0; by < grid.y && !g.failed; ++by)
             for (unsigned bx = 0; bx < grid.x && !g.failed; ++bx) {
                 // LDS content of the previous workgroup is poison, as on the hardware where it is whatever was there
-                memset(g.lds, 0xff, lds_bytes ? lds_bytes : 64);
+                memset(g.lds, 0xff, lds_bytes);
                 for (auto& w : g.waves) {
                     w.live = 0;
                     w.arrived = 0;

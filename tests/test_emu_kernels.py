@@ -39,9 +39,38 @@ for _m in _mods:
 del _fn
 
 
+_PAGE = 4096
+_libc = ctypes.CDLL(None, use_errno=True)
+_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+
+
+def _guarded_copy(t):
+    """A copy of t whose last byte (rounded up to 16) sits right before an inaccessible page: a kernel that reads or
+    writes past the end of an input - what ends in a memory access fault on the GPU - takes a segmentation fault here.
+    FCK_EMU_GUARD=front puts the page in front of the first byte instead (accesses before the start)."""
+    import mmap
+    n = t.numel() * t.element_size()
+    if n == 0:
+        return t.clone()
+    n16 = (n + 15) // 16 * 16
+    total = (n16 + _PAGE - 1) // _PAGE * _PAGE + _PAGE
+    mm = mmap.mmap(-1, total)
+    base = ctypes.addressof(ctypes.c_char.from_buffer(mm))
+    front = os.environ.get("FCK_EMU_GUARD") == "front"
+    guard = base if front else base + total - _PAGE
+    if _libc.mprotect(guard, _PAGE, 0) != 0:   # PROT_NONE
+        raise OSError(ctypes.get_errno(), "mprotect")
+    buf = (ctypes.c_char * n).from_address(base + _PAGE if front else guard - n16)
+    buf._mapping = mm   # the tensor keeps buf alive, buf the mapping
+    out = torch.frombuffer(buf, dtype=torch.uint8, count=n).view(t.dtype).view(t.shape)
+    out.copy_(t.contiguous())
+    return out
+
+
 def _cpu(x, device="cpu"):
-    """stand-in for helpers.dev: a private copy on the CPU (kernels write in place, as they do to device copies)"""
-    return x.clone() if isinstance(x, torch.Tensor) else x
+    """stand-in for helpers.dev: a private copy on the CPU (kernels write in place, as they do to device copies), placed
+    against a guard page"""
+    return _guarded_copy(x) if isinstance(x, torch.Tensor) else x
 
 
 def _wall_timer(fn, cold, repeats):

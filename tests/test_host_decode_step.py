@@ -32,7 +32,7 @@ def cpu_ops(monkeypatch, orc):
 
     def splitkv(q, k, v, num_splits, *, seqlen_k=None, block_table=None, cache_batch_idx=None, cu_seqlens_q=None,
                 cu_seqlens_k=None, max_seqlen_q=0, scale=0.0, mask_type=F.MASK_NONE, window=(-1, -1), o_acc=None,
-                lse_acc=None, decode_variant=0, k_descale=1.0, v_descale=1.0):
+                lse_acc=None, decode_variant=0, k_descale=1.0, v_descale=1.0, max_seqlen_k=0):
         assert decode_variant == 0   # nothing is cached in these tests: the library picks the kernel variant
         calls.append(("splitkv", dict(num_splits=num_splits, mask_type=mask_type, window=tuple(window),
                                       max_seqlen_q=max_seqlen_q, seqlen_k=seqlen_k.clone(), o_acc=o_acc, lse_acc=lse_acc)))

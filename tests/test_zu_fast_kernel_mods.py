@@ -126,3 +126,69 @@ def test_head_pair_decode_with_score_modifiers(fmha, orc, kind, d, page, fp8):
     assert_close(o, ro, 2e-2, f"{kind} on {name.decode()}")
     o1, l1 = fmha.fmha_fwd_splitkv(dev(q), dev(kc), dev(vc), 3, decode_variant=1, **{k: dev(v) for k, v in {**common, **kw}.items()}, **skw)
     assert_close(fmha.fmha_fwd_splitkv_combine(l1, o1, dtype), ro, 2e-2, f"{kind}, one head per workgroup")
+
+
+@pytest.mark.parametrize("variant", [3, 4])
+@pytest.mark.parametrize("d,page", [(128, 128), (64, 64), (128, 32)])
+@pytest.mark.parametrize("ns,bound", [(4, 0), (8, 1500), (3, 700), (1, 0)])
+def test_splits_of_equal_size_for_a_ragged_batch(fmha, orc, variant, d, page, ns, bound):
+    """decode_variant 3 / 4: split s covers keys [s * chunk, (s + 1) * chunk) of every sequence, chunk from the key-count
+    bound and num_splits; short sequences leave their last splits empty; a bound below the longest sequence (700 < 1500)
+    only moves work into the last split.  Partials against the oracle restricted to those ranges, output against the
+    oracle's attention."""
+    g = torch.Generator().manual_seed(ns + d)
+    dtype, hq, hk = torch.bfloat16, 16, 4
+    lens = [1, 31, 32, 33, 500, 1500, 129, 900]
+    kv = gen.paged_kv(lens, hk, d, dtype, g, page)
+    q = gen.randn((len(lens), 1, hq, d), dtype, g)
+    scale = 1 / math.sqrt(d)
+    o_acc, lse_acc = fmha.fmha_fwd_splitkv(dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]), ns, seqlen_k=dev(kv["seqlen_k"]),
+                                           block_table=dev(kv["block_table"]), scale=scale, decode_variant=variant, max_seqlen_k=bound)
+    name = _lib.load().fck_fmha_last_kernel()
+    assert b"equal_chunks" in name and (b"head_pairs" in name) == (variant == 4)
+    o = fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype)
+    ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], scale=scale)
+    assert_close(o, ro, 2e-2, name.decode())
+    # the partial of (sequence b, split s) is attention over its chunk alone
+    capacity = kv["block_table"].shape[1] * page
+    limit = bound if 0 < bound < capacity else capacity
+    chunk = (-(-limit // ns) + 31) // 32 * 32
+    lse = lse_acc.cpu()
+    for b, L in enumerate(lens):
+        for s in range(ns):
+            k0, k1 = min(s * chunk, L), (L if s == ns - 1 else min((s + 1) * chunk, L))
+            if k1 <= k0:
+                assert torch.isinf(lse[b, :, s]).all() and (lse[b, :, s] < 0).all(), (b, s)
+                continue
+            sub = orc.fmha_fwd(q[b:b + 1], kv["k_rows"][b][None, k0:k1].contiguous(), kv["v_rows"][b][None, k0:k1].contiguous(), scale=scale)
+            assert_close(o_acc[b:b + 1, :, s].cpu().permute(0, 2, 1, 3), sub.float(), 2e-2, f"partial of sequence {b}, split {s}")
+
+
+def test_equal_size_splits_refusals_and_tuning(fmha, orc, tmp_path, monkeypatch):
+    from flashck_amd.utils import flags, tuning
+    g = torch.Generator().manual_seed(2)
+    kv = gen.paged_kv([100, 900, 40], 4, 128, torch.bfloat16, g, 48)      # pages of 48 keys: not a multiple of 32
+    q = gen.randn((3, 1, 16, 128), torch.bfloat16, g)
+    with pytest.raises(ValueError, match="splits of equal size"):
+        fmha.fmha_fwd_splitkv(dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]), 2, seqlen_k=dev(kv["seqlen_k"]), block_table=dev(kv["block_table"]),
+                              decode_variant=3)
+    kv = gen.paged_kv([100, 900, 40], 4, 128, torch.bfloat16, g, 128)
+    with pytest.raises(ValueError, match="splits of equal size"):
+        fmha.fmha_fwd_splitkv(dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]), 2, seqlen_k=dev(kv["seqlen_k"]), block_table=dev(kv["block_table"]),
+                              decode_variant=4, logits_soft_cap=2.0)
+    # the tuner can record such a variant, and a later automatic call runs it
+    cache = tuning.TuningCache(str(tmp_path))
+    monkeypatch.setattr(tuning, "default_cache", lambda: cache)
+    flags.set_flag_value("FC_TUNING_NUM_COLD_ITERATION", "1")
+    flags.set_flag_value("FC_TUNING_NUM_REPEATS", "1")
+    try:
+        args = (dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]), dev(kv["seqlen_k"]), dev(kv["block_table"]))
+        rec = fmha.tune_decode_num_splits(*args, max_seqlen_k=900, candidates=(2, 4), variants=(3, 4), cache=cache)
+        assert rec["variant"] in (3, 4) and "equal_chunks" in rec["kernel"]
+        o = fmha.fmha_decode_paged(*args, max_seqlen_k=900)
+        assert b"equal_chunks" in _lib.load().fck_fmha_last_kernel()
+    finally:
+        flags.set_flag_value("FC_TUNING_NUM_COLD_ITERATION", "16")
+        flags.set_flag_value("FC_TUNING_NUM_REPEATS", "64")
+    ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqlen_k=kv["seqlen_k"], block_table=kv["block_table"])
+    assert_close(o, ro, 2e-2, "automatic call with a recorded equal-size variant")
