@@ -179,9 +179,10 @@ def bench_decode(args, torch, fmha, gen, which):
     return res
 
 
-def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=False, kv_fp8=False):
-    """variant: tile variant (fck_fmha_attrs.prefill_variant); alibi: with per-head ALiBi slopes; kv_fp8: K/V cache as e4m3"""
-    w = gen.workload_varlen_prefill(head_dim=d)
+def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=False, kv_fp8=False, dv=None):
+    """variant: tile variant (fck_fmha_attrs.prefill_variant); alibi: with per-head ALiBi slopes; kv_fp8: K/V cache as e4m3;
+    dv: head dim of V / O when it differs from d"""
+    w = gen.workload_varlen_prefill(head_dim=d, v_head_dim=dv)
     dev = "cuda"
     kw = {}
     if alibi:
@@ -191,7 +192,7 @@ def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=Fal
         w["v_cache"] = (w["v_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
         kw.update(k_descale=0.0625, v_descale=0.0625)
     a = [w[k].to(dev) for k in ("q", "k_cache", "v_cache", "cu_seqlens_q", "kv_indptr", "kv_page_indices", "kv_last_page_lens")]
-    o = torch.empty_like(a[0])
+    o = torch.empty(a[0].shape[0], a[0].shape[1], dv or d, dtype=a[0].dtype, device=dev)
 
     def step(i, ev):
         if ev is not None:
@@ -203,10 +204,10 @@ def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=Fal
     wall, kern_ms = time_steps(step, steps, warmup, torch, kernel_events=True)
     from flashck_amd import _lib
     kernel = _lib.load().fck_fmha_last_kernel().decode()
-    flops = gen.prefill_flops(w["lens"], 32, d, d)
-    nbytes = gen.prefill_bytes(w["lens"], 32, 8, d, d)
+    flops = gen.prefill_flops(w["lens"], 32, d, dv or d)
+    nbytes = gen.prefill_bytes(w["lens"], 32, 8, d, dv or d)
     ms = wall / steps * 1e3
-    tag = (" + ALiBi" if alibi else "") + (" [K/V cache fp8 e4m3]" if kv_fp8 else "") + (f" [tile variant {variant}]" if variant else "")
+    tag = (f" (v_head_dim {dv})" if dv else "") + (" + ALiBi" if alibi else "") + (" [K/V cache fp8 e4m3]" if kv_fp8 else "") + (f" [tile variant {variant}]" if variant else "")
     return dict(name=f"varlen causal batch prefill: 16 seqs L~U[128,8192] Hq32/Hk8 D{d} paged P=128 (bf16)" + tag,
                 ms_per_step=ms, flops=flops, bytes=nbytes, tflops=flops / (ms * 1e-3) / 1e12, kernel_ms=kern_ms,
                 kernel_tflops=flops / (kern_ms * 1e-3) / 1e12, total_q=sum(w["lens"]), kernel=kernel)
@@ -379,6 +380,7 @@ def main():
         secondary("prefill_d128_alibi", lambda: prefill(128, alibi=True))
         secondary("prefill_d256_alibi", lambda: prefill(256, alibi=True))
         secondary("prefill_d128_fp8_cache", lambda: prefill(128, kv_fp8=True))
+        secondary("prefill_d192_dv128", lambda: prefill(192, dv=128))
 
     line = {
         "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -571,8 +571,20 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t
         return fail(FCK_ERR_INVALID_ARGUMENT, "prefill_variant %d needs the ping-pong kernel: head dim 64 or 128, query runs longer than 128, "
                                               "pages a multiple of 64 (or no pages), no bias / ALiBi / soft cap / fp8 cache", a.variant);
     if (d_qk != d || dv != d) {
-        // head dims other than 64 / 128 / 256, or qk_head_dim != v_head_dim: the register-staged kernel pads them
+        // Head dims other than 64 / 128 / 256, or qk_head_dim != v_head_dim: every kernel pads them (rows keep their stored
+        // length in memory, the missing columns are zeros in LDS); which kernel follows the rules below, except that an
+        // elementwise bias or a short query run takes the register-staged one.
+        const bool fast = !(a.mod.active() && a.mod.bias_type == FCK_BIAS_ELEMENTWISE);
+        if (fast && d <= 128 && q_max_seq_len > 128) {
+            a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
+            g_kernel = uniform ? "prefill_pp_kernel<uniform_page,padded_head_dim>" : "prefill_pp_kernel<row_lookup,padded_head_dim>";
+            return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+        }
         a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
+        if (fast && d == 256 && uniform) {
+            g_kernel = "prefill_dma_kernel<uniform_page,padded_head_dim>";
+            return launch_status(fck::launch_prefill_dma(a, (int)d, dtype, static_cast<hipStream_t>(stream)), what);
+        }
         g_kernel = uniform ? "prefill_kernel<uniform_page,padded_head_dim>" : "prefill_kernel<row_lookup,padded_head_dim>";
         return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
     }

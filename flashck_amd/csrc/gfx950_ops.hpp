@@ -57,6 +57,11 @@ __device__ __forceinline__ void load_to_lds(uint32_t dst, const void* src)
                  : "memory");
 }
 
+// A lane that sits out a global -> LDS instruction which other lanes of its wave issue (it is masked off for that
+// instruction): nothing to do on the hardware, where the wave's counter of outstanding operations counts the instruction
+// once for all lanes; the emulated twin keeps the lane's own count in step with it.
+#define FCK_LOAD_TO_LDS_MASKED() ((void)0)
+
 // wait until at most N of this wave's vector-memory operations are outstanding (they complete in order)
 template <int N>
 __device__ __forceinline__ void wait_vm()

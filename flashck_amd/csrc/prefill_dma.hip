@@ -38,9 +38,16 @@ __device__ __forceinline__ int k_swz(int row) { return tiles::k_swz<256>(row); }
 __device__ __forceinline__ int v_swz(int row, int lc) { return tiles::v_swz<256>(row, lc); }
 
 // kMod: ALiBi and / or the logits soft cap applied to every score (ArithMod)
-template <typename T, int D, bool kMod = false>
+// kPad: the stored head dims (a.d for Q / K, a.dv for V / O; multiples of 8) are smaller than D: rows are a.d / a.dv
+//   elements apart, a lane whose 16-byte piece lies past a row's end requests nothing and the LDS bytes it would have
+//   filled are zeroed once per workgroup (zero columns of Q and K add nothing to a score, zero columns of V give output
+//   columns that are not stored).  Always together with kMod (the identity when no modifier is set).
+template <typename T, int D, bool kMod = false, bool kPad = false>
 __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a)
 {
+    static_assert(!kPad || kMod, "padded head dims: the general kernel");
+    const int dq = kPad ? a.d : D;    // elements per stored Q / K row
+    const int dvs = kPad ? a.dv : D;  // elements per stored V / O row
     typedef Shape<D> S;
     typedef typename T::vec8 vec8;
     constexpr int BN = S::BN;
@@ -108,12 +115,12 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     // ---- Q fragments (B operand of S^T = K . Q^T): lane (row = l32, k-group = half) ------------------------------
     vec8 qf[S::KT];
     {
-        const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * D +
+        const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * dq +
                              half * 8;
 #pragma unroll
         for (int t = 0; t < S::KT; ++t) {
             u32x4_t v = {0u, 0u, 0u, 0u};
-            if (row_ok) v = ldg16(qp + t * 16);
+            if (row_ok && (!kPad || t * 16 + half * 8 < dq)) v = ldg16(qp + t * 16);
             qf[t] = as_vec8<vec8>(v);
         }
     }
@@ -148,11 +155,44 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     tiles::FirstRows<BN> first_rows{row_lds};
     first_rows.fill(a.kv, ks, t_begin, n, tid, 256);
     auto tile_row0 = [&](int i) __attribute__((always_inline)) -> int64_t { return first_rows.row0(a.kv, ks, t_begin, i, lane); };
+    if constexpr (kPad) {
+        // the LDS bytes no request of this lane will ever fill, in both buffers of each operand
+        const u32x4_t zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int buf = 0; buf < 2; ++buf)
+#pragma unroll
+            for (int u = 0; u < S::LD; ++u) {
+                const int off = (wave + 4 * u) * 1024 + lane * 16;
+                if (((u & 1) ? cp_kc1 : cp_kc0) >= dq) *(u32x4_t FCK_LDS*)(lds + buf * S::TILEB + off) = zero;
+                if (cp_vc >= dvs) *(u32x4_t FCK_LDS*)(lds + (2 + buf) * S::TILEB + off) = zero;
+            }
+    }
     // request this wave's share of the K and V tile i (local index) into buffer buf
     auto request = [&](int i, int buf) __attribute__((always_inline)) {
         const int room = sk_b - 1 - (t_begin + i) * BN;
         const bool whole = room >= BN - 1;  // every row of the tile exists (all tiles but the last of a sequence)
         const int64_t row0 = tile_row0(i);
+        if constexpr (kPad) {
+            // rows are a.d / a.dv elements apart; a piece past the stored row's end is not requested
+#pragma unroll
+            for (int kv = 0; kv < 2; ++kv) {
+                const int64_t rs = (int64_t)a.hk * (kv == 0 ? dq : dvs);
+                const int dim = kv == 0 ? dq : dvs;
+                const uint16_t* tb = (kv == 0 ? kp : vp) + (row0 * rs + hkv * dim);
+                char FCK_LDS* dst0 = lds + ((kv == 0 ? 0 : 2) + buf) * S::TILEB;
+#pragma unroll
+                for (int u = 0; u < S::LD; ++u) {
+                    const int c = kv == 0 ? ((u & 1) ? cp_kc1 : cp_kc0) : cp_vc;
+                    if (c >= dim) {
+                        FCK_LOAD_TO_LDS_MASKED();
+                        continue;
+                    }
+                    const int row = min(cp_row0 + 8 * u, room);  // rows past the last key repeat it (their scores are masked)
+                    tiles::load_to_lds(lds_address(dst0 + (wave + 4 * u) * 1024), tb, (uint32_t)(row * (int)rs + c) * 2u);
+                }
+            }
+            return;
+        }
         const int64_t tile_off = row0 * row_stride + hkv * D;
 #pragma unroll
         for (int kv = 0; kv < 2; ++kv) {
@@ -298,11 +338,14 @@ __global__ __launch_bounds__(256, 1) void prefill_dma_kernel(const PrefillArgs a
     l_run = pair32_sum(l_run);
     if (row_ok) {
         const float inv = (l_run == 0.f) ? 0.f : 1.f / l_run;
-        uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * D;
+        uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * dvs;
 #pragma unroll
         for (int dvb = 0; dvb < S::DVB; ++dvb)
 #pragma unroll
             for (int j4 = 0; j4 < 4; ++j4) {
+                if constexpr (kPad) {
+                    if (dvb * 32 + j4 * 8 + half * 4 >= dvs) continue;
+                }
                 u32x2_t out;
                 out[0] = T::pack2(oacc[dvb][j4 * 4 + 0] * inv, oacc[dvb][j4 * 4 + 1] * inv);
                 out[1] = T::pack2(oacc[dvb][j4 * 4 + 2] * inv, oacc[dvb][j4 * 4 + 3] * inv);
@@ -317,10 +360,9 @@ static hipError_t launch_d(const PrefillArgs& a, hipStream_t st)
     const int g = a.hq / a.hk, gx = (a.batch * a.hk + 7) / 8;
     const dim3 grid(8 * a.m_tiles * gx * g);
     constexpr size_t lds = (size_t)4 * Shape<D>::TILEB + kPrefillPageCache * 4;
-    if (a.mod.active()) {
-        if (a.mod.bias_type == 1) return hipErrorInvalidValue;  // elementwise bias: not in this kernel (the caller routes it away)
-        return launch_with_lds<prefill_dma_kernel<T, D, true>>(grid, dim3(256), lds, st, a);
-    }
+    if (a.mod.bias_type == 1) return hipErrorInvalidValue;  // elementwise bias: not in this kernel (the caller routes it away)
+    if (a.d != D || a.dv != D) return launch_with_lds<prefill_dma_kernel<T, D, true, true>>(grid, dim3(256), lds, st, a);
+    if (a.mod.active()) return launch_with_lds<prefill_dma_kernel<T, D, true>>(grid, dim3(256), lds, st, a);
     return launch_with_lds<prefill_dma_kernel<T, D>>(grid, dim3(256), lds, st, a);
 }
 

@@ -54,11 +54,19 @@ using tiles::v_swz;
 //          multiply per request; the scalar base carries the tile)
 //   bit 1  the per-lane maximum of a tile's raw scores is taken at the end of the matrix phase that produced them,
 //          which shortens the (longer) vector phase by that much; tiles that need masking take it again after the mask
-template <typename T, int D, int BN, bool kUniformPage, bool kMod = false, int kVar = 0>
+// kPad: the stored head dims (a.d for Q / K, a.dv for V / O; multiples of 8) are smaller than D.  Rows are a.d / a.dv
+//   elements apart in memory; a lane whose 16-byte piece lies past a row's end requests nothing, and the LDS bytes it
+//   would have filled are zeroed once per workgroup (the swizzle maps them to the same places in every tile): zero
+//   columns of Q and K add nothing to a score, zero columns of V give output columns that are not stored.  Always
+//   together with kMod (the identity when no modifier is set).
+template <typename T, int D, int BN, bool kUniformPage, bool kMod = false, int kVar = 0, bool kPad = false>
 __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
 {
     constexpr bool kFastRequests = (kVar & 1) != 0, kMaxInMatrixPhase = (kVar & 2) != 0;
     static_assert(kVar == 0 || (kUniformPage && !kMod), "tile variants exist for the plain uniform-page kernel");
+    static_assert(!kPad || kMod, "padded head dims: the general kernel");
+    const int dq = kPad ? a.d : D;    // elements per stored Q / K row
+    const int dvs = kPad ? a.dv : D;  // elements per stored V / O row
     typedef PPShape<D, BN> S;
     typedef typename T::vec8 vec8;
     static_assert(S::NB == 2, "the matrix phase is written for 64-key tiles");
@@ -135,11 +143,11 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     u32x4_t qf[S::KT];
     {
         const uint16_t* qp =
-            reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * D + half * 8;
+            reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * dq + half * 8;
 #pragma unroll
         for (int t = 0; t < S::KT; ++t) {
             qf[t] = u32x4_t{0u, 0u, 0u, 0u};
-            if (row_ok) qf[t] = ldg16(qp + t * 16);
+            if (row_ok && (!kPad || t * 16 + half * 8 < dq)) qf[t] = ldg16(qp + t * 16);
         }
     }
 
@@ -156,6 +164,7 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k);
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v);
     const int64_t row_stride = (int64_t)a.hk * D;
+    const int64_t rs_k = kPad ? (int64_t)a.hk * dq : row_stride, rs_v = kPad ? (int64_t)a.hk * dvs : row_stride;
     const int last_key = sk_b - 1;
 
     // global -> LDS assignment: wave w fills the 1 KiB blocks w, w+8, ... of a tile; lane l of an instruction lands at
@@ -199,7 +208,20 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         for (int u = 0; u < S::LD; ++u) {
             const int row = min(cp_row[u], room);  // rows past the last key repeat it (their scores are masked)
             const uint32_t dst = lds_address(ring + slot_ * S::TILEB + (wave + 8 * u) * 1024);
-            if constexpr (kUniformPage) {
+            if constexpr (kPad) {
+                // rows are a.d / a.dv elements apart; a piece past the stored row's end is not requested (its place in the
+                // tile was zeroed once)
+                const int64_t rs = base == kp ? rs_k : rs_v;
+                const int dim = base == kp ? dq : dvs;
+                if (cp_c[u] >= dim) {
+                    FCK_LOAD_TO_LDS_MASKED();
+                    continue;
+                }
+                if constexpr (kUniformPage)
+                    tiles::load_to_lds(dst, base + (row0 * rs + hkv * dim), (uint32_t)(row * (int)rs + cp_c[u]) * 2u);
+                else
+                    tiles::load_to_lds(dst, base + kv_row(a.kv, ks, kb + row) * rs + hkv * dim + cp_c[u]);
+            } else if constexpr (kUniformPage) {
                 const uint16_t* tb = base + (row0 * row_stride + hkv * D);
                 if (kFastRequests && room >= S::BN - 1)
                     tiles::load_to_lds(dst, tb, cp_off[u]);
@@ -371,6 +393,19 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
         FCK_PIN_VGPR(l_run);
     };
 
+    if constexpr (kPad) {
+        // the LDS bytes no request of this lane will ever fill, in every ring buffer (the same lane and instruction slot of
+        // every tile): nobody else writes them, and the barriers ahead of the first matrix phase publish them
+        const u32x4_t zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int slot_ = 0; slot_ < kRing; ++slot_)
+#pragma unroll
+            for (int u = 0; u < S::LD; ++u) {
+                const int off = slot_ * S::TILEB + (wave + 8 * u) * 1024 + lane * 16;
+                if (cp_k[u] >= dq) *(u32x4_t FCK_LDS*)(k_ring + off) = zero;
+                if (cp_v[u] >= dvs) *(u32x4_t FCK_LDS*)(v_ring + off) = zero;
+            }
+    }
     if (n > 0) {
         typedef std::integral_constant<int, 0> Keep0;
         typedef std::integral_constant<int, 2 * S::LD> KeepBatch;  // one batch = this wave's share of one K and one V tile
@@ -421,11 +456,14 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
     l_run = pair32_sum(l_run);
     if (row_ok) {
         const float inv = (l_run == 0.f) ? 0.f : 1.f / l_run;
-        uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * D;
+        uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * dvs;
 #pragma unroll
         for (int dvb = 0; dvb < S::DVB; ++dvb)
 #pragma unroll
             for (int j4 = 0; j4 < 4; ++j4) {
+                if constexpr (kPad) {
+                    if (dvb * 32 + j4 * 8 + half * 4 >= dvs) continue;
+                }
                 u32x2_t out;
                 out[0] = T::pack2(oacc[dvb][j4 * 4 + 0] * inv, oacc[dvb][j4 * 4 + 1] * inv);
                 out[1] = T::pack2(oacc[dvb][j4 * 4 + 2] * inv, oacc[dvb][j4 * 4 + 3] * inv);
@@ -440,8 +478,12 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
     const int g = a.hq / a.hk, gx = (a.batch * a.hk + 7) / 8;
     const dim3 grid(8 * a.m_tiles * gx * g);
     constexpr size_t lds = (size_t)2 * PPShape<D, BN>::RING * PPShape<D, BN>::TILEB + kPrefillPageCache * 4;
+    if (a.mod.bias_type == 1) return hipErrorInvalidValue;  // elementwise bias: not in this kernel (the caller routes it away)
+    if (a.d != D || a.dv != D) {  // padded head dims
+        if (uniform) return launch_with_lds<prefill_pp_kernel<T, D, BN, true, true, 0, true>>(grid, dim3(512), lds, st, a);
+        return launch_with_lds<prefill_pp_kernel<T, D, BN, false, true, 0, true>>(grid, dim3(512), lds, st, a);
+    }
     if (a.mod.active()) {
-        if (a.mod.bias_type == 1) return hipErrorInvalidValue;  // elementwise bias: not in this kernel (the caller routes it away)
         if (uniform) return launch_with_lds<prefill_pp_kernel<T, D, BN, true, true>>(grid, dim3(512), lds, st, a);
         return launch_with_lds<prefill_pp_kernel<T, D, BN, false, true>>(grid, dim3(512), lds, st, a);
     }

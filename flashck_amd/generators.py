@@ -141,13 +141,13 @@ def workload_appendkv_decode(seed=BASE_SEED + 4, batch=16, hq=32, hk=8, head_dim
 
 
 def workload_varlen_prefill(seed=BASE_SEED + 5, batch=16, hq=32, hk=8, head_dim=128, min_len=128, max_len=8192,
-                            page_size=128, dtype=torch.bfloat16, lens=None):
+                            page_size=128, dtype=torch.bfloat16, lens=None, v_head_dim=None):
     """5: varlen causal batch prefill, sq = sk = L_b packed by cu_seqlens, K/V in a shuffled paged cache.
-    `lens` fixes the lengths instead of drawing them."""
+    `lens` fixes the lengths instead of drawing them; `v_head_dim` is the head dim of V when it differs from Q / K's."""
     g = _gen(seed)
     lens = list(lens) if lens is not None else randint_list(min_len, max_len, batch, g)
     batch = len(lens)
-    kv = paged_kv(lens, hk, head_dim, dtype, g, page_size)
+    kv = paged_kv(lens, hk, head_dim, dtype, g, page_size, dv=v_head_dim)
     cu = torch.zeros(batch + 1, dtype=torch.int32)
     cu[1:] = torch.tensor(lens).cumsum(0)
     total = int(cu[-1])

@@ -185,7 +185,7 @@ bool late_loads()
 void request_copy(char* dst, const char* src)
 {
     if (!late_loads()) {
-        memcpy(dst, src, 16);
+        if (dst) memcpy(dst, src, 16);
         return;
     }
     Lane& l = *cur;
@@ -199,7 +199,7 @@ void land_copies(int keep)
     Lane& l = *cur;
     while (l.pending_count > keep) {
         const PendingCopy& c = l.pending[l.pending_head];
-        memcpy(c.dst, c.src, 16);
+        if (c.dst) memcpy(c.dst, c.src, 16);  // null: the lane was masked off for this instruction
         l.pending_head = (l.pending_head + 1) & 255;
         --l.pending_count;
     }

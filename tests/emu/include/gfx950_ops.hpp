@@ -40,6 +40,9 @@ inline void load_to_lds(uint32_t dst, const void* base, uint32_t off)
 }
 inline void load_to_lds(uint32_t dst, const void* src) { emu::request_copy((char*)(uintptr_t)dst + emu::cur->lane * 16, (const char*)src); }
 
+// a masked-off lane of an issued instruction: an empty entry in the lane's queue
+#define FCK_LOAD_TO_LDS_MASKED() emu::request_copy(nullptr, nullptr)
+
 // the kernels count only their own global -> LDS instructions; so does this
 template <int N>
 inline void wait_vm()

@@ -192,3 +192,41 @@ def test_equal_size_splits_refusals_and_tuning(fmha, orc, tmp_path, monkeypatch)
         flags.set_flag_value("FC_TUNING_NUM_REPEATS", "64")
     ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqlen_k=kv["seqlen_k"], block_table=kv["block_table"])
     assert_close(o, ro, 2e-2, "automatic call with a recorded equal-size variant")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d,dv,page", [(96, 96, 128), (40, 72, 64), (48, 64, 64), (128, 64, 48), (192, 128, 64), (160, 256, 128), (256, 136, 64),
+                                       (8, 8, 64)])
+@pytest.mark.parametrize("kind", ["none", "alibi_cap"])
+def test_padded_head_dims_on_the_fast_kernels(fmha, orc, dtype, d, dv, page, kind):
+    """qk_head_dim != v_head_dim and head dims between the instantiated ones, on long query runs: rows keep their stored
+    length in memory, the missing columns are zeros in LDS (written once per workgroup) and are never requested."""
+    g = torch.Generator().manual_seed(d * 3 + dv)
+    hq, hk, lens = 4, 2, [300, 700, 129, 1]
+    kv = gen.paged_kv(lens, hk, d, dtype, g, page, dv=dv)
+    cu = torch.tensor([0, 300, 1000, 1129, 1130], dtype=torch.int32)
+    q = gen.randn((1130, hq, d), dtype, g)
+    kw = {} if kind == "none" else _mods(kind, hq, 4, g)
+    scale = 1 / math.sqrt(d)
+    o = fmha.fmha_fwd_pagedkv(dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]), dev(kv["seqlen_k"]), dev(kv["block_table"]), cu_seqlens_q=dev(cu),
+                              max_seqlen_q=700, scale=scale, mask_type=2, window=(-1, 0), **{k: dev(v) for k, v in kw.items()})
+    name = _lib.load().fck_fmha_last_kernel()
+    big = max(d, dv) > 128
+    if big:
+        assert name == b"prefill_dma_kernel<uniform_page,padded_head_dim>"
+    else:
+        assert name == (b"prefill_pp_kernel<uniform_page,padded_head_dim>" if page % 64 == 0 else b"prefill_pp_kernel<row_lookup,padded_head_dim>")
+    assert tuple(o.shape) == (1130, hq, dv)
+    ro = orc.fmha_fwd(q, kv["k_cache"], kv["v_cache"], seqstart_q=cu, seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], scale=scale,
+                      mask_type=2, window=(-1, 0), **kw)
+    assert_close(o, ro, ATOL[dtype], f"({d}, {dv}) on {name.decode()}")
+
+
+def test_padded_head_dims_dense_batch_mode(fmha, orc):
+    g = torch.Generator().manual_seed(41)
+    for d, dv in ((192, 128), (80, 80)):
+        q, k, v = gen.randn((2, 200, 4, d), torch.bfloat16, g), gen.randn((2, 260, 2, d), torch.bfloat16, g), gen.randn((2, 260, 2, dv), torch.bfloat16, g)
+        o = fmha.fmha_fwd(dev(q), dev(k), dev(v), mask_type=2, window=(-1, 0))
+        assert b"padded_head_dim" in _lib.load().fck_fmha_last_kernel() and b"prefill_kernel" not in _lib.load().fck_fmha_last_kernel()
+        ro = orc.fmha_fwd(q, k, v, mask_type=2, window=(-1, 0))
+        assert_close(o, ro, 2e-2, f"dense ({d}, {dv})")
