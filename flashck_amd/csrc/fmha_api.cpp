@@ -175,6 +175,29 @@ int cu_count()
     return cus[dev];
 }
 
+// The slice of the fused entry point's device array that `stream` uses on the current device: the one it was given on
+// its first call, else the first free one; -1 when kDecodeScratchSlices other streams hold them all.  forget: empty the
+// current device's table instead (returns 0).  Host memory only; a stream handle is just a key here, never dereferenced.
+int fused_slice(hipStream_t stream, bool forget)
+{
+    constexpr int kMaxDev = 64;
+    static std::mutex mu;
+    static hipStream_t owner[kMaxDev][fck::kDecodeScratchSlices];
+    static int used[kMaxDev];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return -1;
+    std::lock_guard<std::mutex> lock(mu);
+    if (forget) {
+        used[dev] = 0;
+        return 0;
+    }
+    for (int i = 0; i < used[dev]; ++i)
+        if (owner[dev][i] == stream) return i;
+    if (used[dev] == fck::kDecodeScratchSlices) return -1;
+    owner[dev][used[dev]] = stream;
+    return used[dev]++;
+}
+
 }  // namespace
 
 extern "C" {
@@ -393,8 +416,15 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
                     (long)fck::kDecodeScratchTickets, (long)tickets);
     float* scratch = nullptr;
     if (hipError_t e = fck::decode_scratch(&scratch); e != hipSuccess) return launch_status(e, "scratch symbol lookup");
-    a.tickets = reinterpret_cast<uint32_t*>(scratch);
-    a.o_acc = scratch + fck::kDecodeScratchTickets;
+    const int slice = fused_slice(static_cast<hipStream_t>(stream), false);
+    if (slice < 0)
+        return fail(FCK_ERR_UNSUPPORTED,
+                    "the fused split-KV entry point serves at most %d streams per GPU (each owns a slice of the library's device "
+                    "array); use one of them, or fck_fmha_fused_reset once no fused call is in flight, or fck_fmha_fwd_splitkv + "
+                    "fck_fmha_fwd_splitkv_combine with a caller-owned workspace",
+                    fck::kDecodeScratchSlices);
+    a.tickets = reinterpret_cast<uint32_t*>(scratch) + slice * fck::kDecodeScratchTickets;
+    a.o_acc = scratch + fck::kDecodeScratchSlices * fck::kDecodeScratchTickets + slice * fck::kDecodeScratchPartialFloats;
     a.lse_acc = a.o_acc + part_rows * dv;
     a.o = o;
     int hpw = 1;
@@ -408,7 +438,9 @@ int fck_fmha_fused_reset(void* stream)
     g_err[0] = 0;
     float* scratch = nullptr;
     if (hipError_t e = fck::decode_scratch(&scratch); e != hipSuccess) return launch_status(e, "scratch symbol lookup");
-    return launch_status(fck::launch_clear_tickets(reinterpret_cast<uint32_t*>(scratch), (int)fck::kDecodeScratchTickets, static_cast<hipStream_t>(stream)),
+    fused_slice(nullptr, true);
+    return launch_status(fck::launch_clear_tickets(reinterpret_cast<uint32_t*>(scratch),
+                                                   (int)(fck::kDecodeScratchSlices * fck::kDecodeScratchTickets), static_cast<hipStream_t>(stream)),
                          "ticket reset launch");
 }
 

@@ -123,9 +123,13 @@ hipError_t launch_clear_tickets(uint32_t* tickets, int n, hipStream_t st);
 hipError_t launch_splitkv_decode(const SplitKvArgs& a, int d, int dtype, int rows_max, bool uniform_page, int num_cu,
                                  hipStream_t st, int* heads_per_workgroup = nullptr);
 // Device memory the fused split-KV entry point uses instead of a caller-owned workspace: a fixed array in the library
-// (one copy per GPU): kDecodeScratchTickets arrival counters (self-resetting), then the partial results.
+// (one copy per GPU), cut into kDecodeScratchSlices equal slices so that calls on different streams of a GPU never share
+// one (a stream keeps the slice it got on its first call).  Layout: the arrival counters of all slices
+// (kDecodeScratchTickets each, self-resetting), then the partial results of all slices (kDecodeScratchPartialFloats each).
 constexpr int64_t kDecodeScratchTickets = 16384;
 constexpr int64_t kDecodeScratchPartialFloats = (int64_t)4 << 20;  // 16 MiB
+constexpr int kDecodeScratchSlices = 4;
+constexpr int64_t kDecodeScratchFloats = kDecodeScratchSlices * (kDecodeScratchTickets + kDecodeScratchPartialFloats);
 // address of the array on the current device (looked up once per device)
 hipError_t decode_scratch(float** ptr);
 // row tiles per (sequence, KV head) the split-KV launcher uses for `rows_max` packed query rows

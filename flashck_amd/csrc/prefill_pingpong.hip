@@ -210,7 +210,10 @@ __global__ __launch_bounds__(512) void prefill_pp_kernel(const PrefillArgs a)
             const uint32_t dst = lds_address(ring + slot_ * S::TILEB + (wave + 8 * u) * 1024);
             if constexpr (kPad) {
                 // rows are a.d / a.dv elements apart; a piece past the stored row's end is not requested (its place in the
-                // tile was zeroed once)
+                // tile was zeroed once).  The waits below count instructions per wave, so every one of the S::LD
+                // instructions must still be issued by every wave: it is, because a 1 KiB block holds whole rows, the
+                // swizzle only permutes the pieces of a row, and piece 0 of a row is always stored (dim >= 8), so no
+                // instruction has all its lanes skipped.
                 const int64_t rs = base == kp ? rs_k : rs_v;
                 const int dim = base == kp ? dq : dvs;
                 if (cp_c[u] >= dim) {

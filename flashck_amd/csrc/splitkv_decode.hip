@@ -563,7 +563,7 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
 // ------------------------------------------------------------------------------------------------------
 // Workspace of the fused entry point.  In host code the array's name is only a handle: its device address is looked up
 // per device with hipGetSymbolAddress, and only that address is ever handed to a kernel.
-static __device__ __align__(256) float g_decode_scratch[kDecodeScratchTickets + kDecodeScratchPartialFloats];
+static __device__ __align__(256) float g_decode_scratch[kDecodeScratchFloats];
 
 hipError_t decode_scratch(float** ptr)
 {

@@ -223,8 +223,9 @@ def _debug_validate(**kw):
 
 
 def fused_reset() -> None:
-    """Zero the arrival tickets of fmha_fwd_splitkv_fused on the current device (after a fused launch that did not run
-    to completion; see fck_fmha_fused_reset)."""
+    """Zero the arrival tickets of fmha_fwd_splitkv_fused on the current device and forget which stream owns which slice
+    of the library's array (after a fused launch that did not run to completion, or to serve other streams; only while
+    no fused call is in flight; see fck_fmha_fused_reset)."""
     _call("fck_fmha_fused_reset", _stream())
 
 
@@ -400,7 +401,9 @@ def fmha_fwd_splitkv_fused(q, k, v, num_splits: int = 0, *, seqlen_k=None, block
     """Split-KV forward + LSE combine in one launch that allocates nothing on the GPU side: the partial results live in
     a fixed device array of the library (limits: see fused_splitkv_fits; beyond them NotImplementedError).
 
-    num_splits = 0 lets the library take its heuristic split count for the CU count and the longest possible KV length.  Calls that overlap in time on one GPU (different streams) race on that array; calls on one stream are safe.
+    num_splits = 0 lets the library take its heuristic split count for the CU count and the longest possible KV length.
+    Each stream owns a slice of that array from its first call on; at most 4 streams per GPU (then NotImplementedError
+    until fused_reset()).
     Arguments as fmha_fwd_splitkv; returns o [B,sq,Hq,Dv] (or [total_q,Hq,Dv] in group mode).
     """
     group = cu_seqlens_q is not None

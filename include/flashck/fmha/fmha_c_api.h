@@ -190,11 +190,16 @@ FCK_EXPORT int fck_fmha_fwd_splitkv_attrs(const void* q, const void* k, const vo
  * launch FmhaFwdSplitKV and FmhaFwdSplitKVCombine separately); it is for callers that cannot allocate or want a single
  * launch: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  *
- * The partial results go to a fixed device array inside the library (one copy per GPU, 16 MiB + 64 KiB, held until
- * the process ends) and the workgroup that delivers the last partial result of a (sequence, KV-head group) merges
- * the splits and writes `o`.  Limits: Bs * Hq * num_splits * Sq * (Dv + 1) <= 4 Mi floats and
- * B * Hk * row_tiles <= 16384, else FCK_ERR_UNSUPPORTED (nothing is launched).  All calls on one GPU share the array:
- * calls that overlap in time on one GPU (different streams, different threads) race; calls on one stream are safe.
+ * The partial results go to a fixed device array inside the library (one copy per GPU, 4 slices of 16 MiB + 64 KiB,
+ * held until the process ends) and the workgroup that delivers the last partial result of a (sequence, KV-head group)
+ * merges the splits and writes `o`.  Limits: Bs * Hq * num_splits * Sq * (Dv + 1) <= 4 Mi floats and
+ * B * Hk * row_tiles <= 16384, else FCK_ERR_UNSUPPORTED (nothing is launched).
+ *
+ * A stream owns one slice of the array on its GPU from its first fused call on, so calls on up to 4 different streams
+ * of a GPU may overlap in time; a fifth stream is refused with FCK_ERR_UNSUPPORTED (nothing is launched) until
+ * fck_fmha_fused_reset has forgotten the owners.  Calls on one stream are ordered by the stream, from whichever host
+ * threads they come.  What still races: one captured graph replayed on two streams at once (its slice was fixed at
+ * capture).
  *
  * num_splits > 0: that many equal key ranges, exactly as fck_fmha_fwd_splitkv.  num_splits == 0: the library takes
  * fck_fmha_num_splits_heuristic of the CU count and the longest possible KV length (the block table's capacity, else
@@ -211,11 +216,12 @@ FCK_EXPORT int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const vo
                                           int32_t dtype, void* stream);
 
 /*
- * Puts the arrival tickets of fck_fmha_fwd_splitkv_fused back to zero on the current device (one small fill launch on
- * `stream`, nothing allocated).  The tickets reset themselves at the end of every fused launch that runs to
- * completion; after a launch that did not (a device error, a cancelled graph launch) they may be left non-zero and
- * every later fused call on that GPU would merge at the wrong moment: call this once before going on.  No counterpart
- * in the reference.
+ * Puts the arrival tickets of fck_fmha_fwd_splitkv_fused (of every slice) back to zero on the current device (one small
+ * fill launch on `stream`, nothing allocated) and forgets which stream owns which slice.  The tickets reset themselves
+ * at the end of every fused launch that runs to completion; after a launch that did not (a device error, a cancelled
+ * graph launch) they may be left non-zero and every later fused call on that slice would merge at the wrong moment:
+ * call this once before going on.  Also the way to hand the slices to other streams.  Call it only when no fused call
+ * is in flight on the GPU, and order later fused calls after `stream`'s fill.  No counterpart in the reference.
  */
 FCK_EXPORT int fck_fmha_fused_reset(void* stream);
 

@@ -96,3 +96,59 @@ def test_fused_rejects_what_does_not_fit():
     rc = lib.fck_fmha_fwd_splitkv_fused(_vp(x), _vp(x), _vp(x), None, _vp(x), None, None, _vp(i), _vp(i), None, 64, 1, 0, 64, 8,
                                         128, 128, 1, 128, 64 * 4, 128, 0.1, -1, -1, 0, 4, _stream())
     assert rc == -2 and b"at most" in lib.fck_last_error()
+
+
+def _other_streams(n):
+    """n stream handles besides the current one, and whatever keeps them alive: torch streams on a GPU; under the CPU
+    emulator (which runs every launch at once and never looks at the handle) distinct made-up handles."""
+    if helpers.DEVICE == "cpu":
+        return [ctypes.c_void_p(0x1000 * (i + 1)) for i in range(n)], None
+    streams = [torch.cuda.Stream() for _ in range(n)]
+    return [ctypes.c_void_p(s.cuda_stream) for s in streams], streams
+
+
+def test_fused_streams_own_slices():
+    """Each stream gets a slice of the library's array of its own: four streams are served (every call equal to the
+    two-launch path), a fifth is refused without a launch, and after fck_fmha_fused_reset it is served."""
+    lib = _lib.load()
+    assert lib.fck_fmha_fused_reset(_stream()) == 0, lib.fck_last_error().decode()
+    torch.cuda.synchronize()
+    g = torch.Generator().manual_seed(79)
+    handles, keep = _other_streams(5)
+    kv = gen.paged_kv([700, 31, 1500, 260], 4, 128, torch.bfloat16, g, 64)
+    q = gen.randn((4, 1, 16, 128), torch.bfloat16, g)
+    B, Hq, D, Hk, page, ns = 4, 16, 128, 4, 64, 3
+    qd, kc, vc, sl, bt = dev(q), dev(kv["k_cache"]), dev(kv["v_cache"]), dev(kv["seqlen_k"]), dev(kv["block_table"])
+    _, o_ref = _run_both(lib, kv, q, ns)  # the current stream takes the first slice
+    torch.cuda.synchronize()
+
+    def fused_on(handle, out):
+        return lib.fck_fmha_fwd_splitkv_fused(_vp(qd), _vp(kc), _vp(vc), None, _vp(out), None, None, _vp(sl), _vp(bt), None, B, 1, 0,
+                                              Hq, Hk, D, D, 1, ns, bt.numel(), page, 1.0 / math.sqrt(D), -1, -1, 0, 4, handle)
+
+    outs = [torch.full(q.shape, float("nan"), dtype=q.dtype, device=helpers.DEVICE) for _ in handles]
+    torch.cuda.synchronize()  # the fills ran on the current stream; the calls below run on others
+    # three more streams, launched back to back without a wait between them, twice each
+    for _ in range(2):
+        for h, o in zip(handles[:3], outs[:3]):
+            assert fused_on(h, o) == 0, lib.fck_last_error().decode()
+    torch.cuda.synchronize()
+    for i in range(3):
+        assert_bits_equal(outs[i], o_ref, f"stream {i + 1}")
+    # all four slices are owned now
+    assert fused_on(handles[3], outs[3]) == -2 and b"streams per GPU" in lib.fck_last_error()
+    torch.cuda.synchronize()
+    assert torch.isnan(outs[3].float()).all(), "a refused call must not launch"
+    # the owners still work after the refusal
+    assert fused_on(handles[0], outs[0]) == 0, lib.fck_last_error().decode()
+    torch.cuda.synchronize()
+    assert lib.fck_fmha_fused_reset(_stream()) == 0, lib.fck_last_error().decode()
+    torch.cuda.synchronize()
+    for h, o in zip(handles[3:], outs[3:]):
+        assert fused_on(h, o) == 0, lib.fck_last_error().decode()
+    torch.cuda.synchronize()
+    for i in (3, 4):
+        assert_bits_equal(outs[i], o_ref, f"stream {i + 1} after the reset")
+    assert lib.fck_fmha_fused_reset(_stream()) == 0  # leave the table empty for whoever comes next
+    torch.cuda.synchronize()
+    del keep
