@@ -138,14 +138,18 @@ def bench_decode(args, torch, fmha, gen, which):
     dev = "cuda"
     q = w["q"].to(dev)
     bt, sl = w["block_table"].to(dev), w["seqlen_k"].to(dev)
-    kv_fp8 = getattr(args, "kv_fp8", False)
+    all_fp8 = getattr(args, "all_fp8", False)  # Q, P and O in e4m3 as well (the query scale goes into the softmax scale)
+    kv_fp8 = getattr(args, "kv_fp8", False) or all_fp8
     scales = {}
+    if all_fp8:
+        q = (q.float() / 0.0625).to(torch.float8_e4m3fn)
+        w["scale"] = w["scale"] * 0.0625
     if kv_fp8:
         # unit-variance data: a static scale of 1/16 keeps it well inside the e4m3 range (+-448)
         scales = dict(k_descale=0.0625, v_descale=0.0625)
         w["k_cache"] = (w["k_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
         w["v_cache"] = (w["v_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
-        name += " [K/V cache fp8 e4m3]"
+        name += " [Q, K, V, P, O fp8 e4m3]" if all_fp8 else " [K/V cache fp8 e4m3]"
     pools = [(w["k_cache"].to(dev), w["v_cache"].to(dev))]
     for _ in range(args.copies - 1):
         pools.append((pools[0][0].clone(), pools[0][1].clone()))
@@ -179,12 +183,16 @@ def bench_decode(args, torch, fmha, gen, which):
     return res
 
 
-def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=False, kv_fp8=False, dv=None):
+def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=False, kv_fp8=False, dv=None, all_fp8=False):
     """variant: tile variant (fck_fmha_attrs.prefill_variant); alibi: with per-head ALiBi slopes; kv_fp8: K/V cache as e4m3;
-    dv: head dim of V / O when it differs from d"""
+    all_fp8: Q, P and O in e4m3 as well; dv: head dim of V / O when it differs from d"""
     w = gen.workload_varlen_prefill(head_dim=d, v_head_dim=dv)
     dev = "cuda"
     kw = {}
+    kv_fp8 = kv_fp8 or all_fp8
+    if all_fp8:
+        w["q"] = (w["q"].float() / 0.0625).to(torch.float8_e4m3fn)
+        w["scale"] = w["scale"] * 0.0625
     if alibi:
         kw["alibi_slopes"] = (torch.arange(1, 33, dtype=torch.float32) / 256).to(dev)
     if kv_fp8:
@@ -207,7 +215,7 @@ def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=Fal
     flops = gen.prefill_flops(w["lens"], 32, d, dv or d)
     nbytes = gen.prefill_bytes(w["lens"], 32, 8, d, dv or d)
     ms = wall / steps * 1e3
-    tag = (f" (v_head_dim {dv})" if dv else "") + (" + ALiBi" if alibi else "") + (" [K/V cache fp8 e4m3]" if kv_fp8 else "") + (f" [tile variant {variant}]" if variant else "")
+    tag = (f" (v_head_dim {dv})" if dv else "") + (" + ALiBi" if alibi else "") + (" [Q, K, V, P, O fp8 e4m3]" if all_fp8 else " [K/V cache fp8 e4m3]" if kv_fp8 else "") + (f" [tile variant {variant}]" if variant else "")
     return dict(name=f"varlen causal batch prefill: 16 seqs L~U[128,8192] Hq32/Hk8 D{d} paged P=128 (bf16)" + tag,
                 ms_per_step=ms, flops=flops, bytes=nbytes, tflops=flops / (ms * 1e-3) / 1e12, kernel_ms=kern_ms,
                 kernel_tflops=flops / (kern_ms * 1e-3) / 1e12, total_q=sum(w["lens"]), kernel=kernel)
@@ -359,9 +367,9 @@ def main():
             out.update(variant=best, tried_kernel_ms={k: t["ms"] for k, t in tried.items()})
             return out
 
-        def splitkv_variant(path, ns, kv_fp8=False):
+        def splitkv_variant(path, ns, kv_fp8=False, all_fp8=False):
             a2 = argparse.Namespace(**vars(args))
-            a2.steps, a2.warmup, a2.decode_path, a2.num_splits, a2.kv_fp8 = max(20, args.steps // 2), 10, path, ns, kv_fp8
+            a2.steps, a2.warmup, a2.decode_path, a2.num_splits, a2.kv_fp8, a2.all_fp8 = max(20, args.steps // 2), 10, path, ns, kv_fp8, all_fp8
             r3 = bench_decode(a2, torch, fmha, gen, "splitkv")
             return dict(workload=r3["name"], us_per_call=r3["ms_per_step"] * 1e3, gbs=r3["gbs"],
                         pct_of_hbm_peak=100 * r3["gbs"] / HBM_PEAK_GBS, kernel_us=r3["kernel_ms"] * 1e3, num_splits=r3["num_splits"])
@@ -371,6 +379,7 @@ def main():
         secondary("splitkv_library_splits", lambda: splitkv_variant("two-launch", ns_lib))
         secondary("splitkv_fused", lambda: splitkv_variant("fused", 0))
         secondary("splitkv_fp8_cache", lambda: splitkv_variant("two-launch", ns_lib, kv_fp8=True))
+        secondary("splitkv_all_fp8", lambda: splitkv_variant("two-launch", ns_lib, all_fp8=True))
         secondary("paged_decode", paged)
         secondary("paged_decode_tuned", paged_tuned)
         secondary("appendkv", append)
@@ -380,6 +389,7 @@ def main():
         secondary("prefill_d128_alibi", lambda: prefill(128, alibi=True))
         secondary("prefill_d256_alibi", lambda: prefill(256, alibi=True))
         secondary("prefill_d128_fp8_cache", lambda: prefill(128, kv_fp8=True))
+        secondary("prefill_d128_all_fp8", lambda: prefill(128, all_fp8=True))
         secondary("prefill_d192_dv128", lambda: prefill(192, dv=128))
 
     line = {

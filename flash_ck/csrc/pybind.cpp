@@ -30,10 +30,16 @@ void* current_stream() { return static_cast<void*>(c10::hip::getCurrentHIPStream
 constexpr bool kHostTensors = false;
 #endif
 
+// float8_e4m3fn: the all-fp8 roles (Q, K, V, P and O in e4m3), where the library has kernels for them
+int32_t dtype_id(at::ScalarType t)
+{
+    TORCH_CHECK(t == at::kHalf || t == at::kBFloat16 || t == at::kFloat8_e4m3fn, "FMHA supports float16, bfloat16 and float8_e4m3fn, got ", t);
+    return t == at::kHalf ? FCK_DTYPE_FP16 : t == at::kBFloat16 ? FCK_DTYPE_BF16 : FCK_DTYPE_FP8;
+}
+
 int32_t dtype_id(const Tensor& t)
 {
-    TORCH_CHECK(t.scalar_type() == at::kHalf || t.scalar_type() == at::kBFloat16, "FMHA supports float16 and bfloat16, got ", t.scalar_type());
-    return t.scalar_type() == at::kHalf ? FCK_DTYPE_FP16 : FCK_DTYPE_BF16;
+    return dtype_id(t.scalar_type());
 }
 
 void check_gpu(const Tensor& t, const char* name, int64_t ndim = -1)
@@ -135,7 +141,7 @@ Tensor fmha_fwd_splitkv_combine(const Tensor& lse_acc, const Tensor& o_acc, at::
     check_gpu(lse_acc, "lse_acc", 4);
     check_gpu(o_acc, "o_acc", 5);
     TORCH_CHECK(lse_acc.scalar_type() == at::kFloat && o_acc.scalar_type() == at::kFloat, "the partials are float32");
-    TORCH_CHECK(dtype == at::kHalf || dtype == at::kBFloat16, "the output is float16 or bfloat16");
+    const int32_t out_dtype = dtype_id(dtype);
     const int64_t bs = o_acc.size(0), Hq = o_acc.size(1), ns = o_acc.size(2), sq = o_acc.size(3), Dv = o_acc.size(4);
     TORCH_CHECK(lse_acc.sizes() == at::IntArrayRef({bs, Hq, ns, sq}), "lse_acc does not match o_acc");
     const bool group = cu_seqlens_q.has_value();
@@ -143,7 +149,7 @@ Tensor fmha_fwd_splitkv_combine(const Tensor& lse_acc, const Tensor& o_acc, at::
     Tensor o = group ? at::empty({sq, Hq, Dv}, o_acc.options().dtype(dtype)) : at::empty({bs, sq, Hq, Dv}, o_acc.options().dtype(dtype));
     check(fck_fmha_fwd_splitkv_combine(lse_acc.data_ptr(), o_acc.data_ptr(), o.data_ptr(), index_ptr(cu_seqlens_q, "cu_seqlens_q"),
                                        group ? cu_seqlens_q->numel() - 1 : bs, sq, Hq, Dv, max_seqlen_q > 0 ? max_seqlen_q : sq, ns,
-                                       dtype == at::kHalf ? FCK_DTYPE_FP16 : FCK_DTYPE_BF16, current_stream()),
+                                       out_dtype, current_stream()),
           "fmha_fwd_splitkv_combine");
     return o;
 }

@@ -18,7 +18,7 @@ class Attrs(ctypes.Structure):
                 ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64),
                 ("logits_soft_cap", ctypes.c_float), ("kv_dtype", ctypes.c_int32), ("k_descale", ctypes.c_float),
                 ("v_descale", ctypes.c_float), ("decode_variant", ctypes.c_int32), ("prefill_variant", ctypes.c_int32),
-                ("bias_cols", ctypes.c_int64), ("max_seqlen_k", ctypes.c_int64)]
+                ("bias_cols", ctypes.c_int64), ("max_seqlen_k", ctypes.c_int64), ("o_scale", ctypes.c_float)]
 
 
 _ap = ctypes.POINTER(Attrs)

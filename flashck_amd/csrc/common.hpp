@@ -149,6 +149,23 @@ __device__ __forceinline__ uint32_t f32_to_fp8_sat(float x)
     return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xffu;
 }
 
+// two fp32 values in [0, 448] rounded to the nearest e4m3 value (ties to even), as fp32 again
+__device__ __forceinline__ f32x2_t round_to_fp8(float a, float b)
+{
+    return __builtin_amdgcn_cvt_pk_f32_fp8(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false), false);
+}
+
+// four fp32 values -> four e4m3 bytes (a in the lowest), each converted as f32_to_fp8_sat does
+__device__ __forceinline__ uint32_t pack_fp8x4_sat(float a, float b, float c, float d)
+{
+    auto clamp = [](float x) {
+        const bool finite = (__builtin_bit_cast(uint32_t, x) & 0x7f800000u) != 0x7f800000u;
+        return finite ? fminf(fmaxf(x, -448.f), 448.f) : x;
+    };
+    const int lo = __builtin_amdgcn_cvt_pk_fp8_f32(clamp(a), clamp(b), 0, false);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(clamp(c), clamp(d), lo, true);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

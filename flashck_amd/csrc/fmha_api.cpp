@@ -18,13 +18,13 @@ namespace {
 thread_local char g_err[512] = "";
 thread_local const char* g_kernel = "";  // kernel family of the calling thread's last launch
 
-// "splitkv_decode_kernel<uniform_page|row_lookup[,head_pairs][,kv_fp8][,score_mod][,padded_head_dim][,fused][,equal_chunks]>": the
+// "splitkv_decode_kernel<uniform_page|row_lookup[,head_pairs][,kv_fp8|,all_fp8][,score_mod][,padded_head_dim][,fused][,equal_chunks]>": the
 // variant the calling thread's last split-KV launch took
-void name_decode_kernel(bool uniform, int heads_per_workgroup, bool kv8, bool mod, bool padded, bool fused, bool chunks)
+void name_decode_kernel(bool uniform, int heads_per_workgroup, bool kv8, bool mod, bool padded, bool fused, bool chunks, bool q8 = false)
 {
     thread_local char name[128];
     snprintf(name, sizeof(name), "splitkv_decode_kernel<%s%s%s%s%s%s%s>", uniform ? "uniform_page" : "row_lookup",
-             heads_per_workgroup == 2 ? ",head_pairs" : "", kv8 ? ",kv_fp8" : "", mod && !padded ? ",score_mod" : "",
+             heads_per_workgroup == 2 ? ",head_pairs" : "", q8 ? ",all_fp8" : kv8 ? ",kv_fp8" : "", mod && !padded ? ",score_mod" : "",
              padded ? ",padded_head_dim" : "", fused ? ",fused" : "", chunks ? ",equal_chunks" : "");
     g_kernel = name;
 }
@@ -40,8 +40,10 @@ int fail(int code, const char* fmt, ...)
 
 int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, int32_t dtype)
 {
-    if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16)
-        return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
+    if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16 && dtype != FCK_DTYPE_FP8)
+        return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT8 (1, e4m3), FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
+    if (dtype == FCK_DTYPE_FP8 && (d != dv || (d != 64 && d != 128 && d != 256)))
+        return fail(FCK_ERR_UNSUPPORTED, "e4m3 queries need qk_head_dim = v_head_dim in {64, 128, 256}");
     if (batch <= 0 || hq <= 0 || hk <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch and head counts must be positive");
     if (hq % hk != 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_num_heads %ld is not a multiple of kv_num_heads %ld", (long)hq, (long)hk);
     // Kernels are built for head dims 64, 128 and 256; any other qk_head_dim / v_head_dim (the two may differ) that is a
@@ -49,6 +51,28 @@ int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, i
     // is_pad_qk_head_dim / is_pad_v_head_dim traits, fmha_fwd_split_kv_codegen.h:106-107).
     if (d < 8 || dv < 8 || d > 256 || dv > 256 || d % 8 || dv % 8)
         return fail(FCK_ERR_UNSUPPORTED, "qk_head_dim %ld / v_head_dim %ld: head dims are multiples of 8 in [8, 256]", (long)d, (long)dv);
+    return FCK_OK;
+}
+
+// Type the kernels compute a call in.  The all-fp8 roles (Q, K, V, P and O in e4m3) run on the bf16 instantiations: every
+// e4m3 value is a bf16 value, so widening the operands is exact, and P is rounded to e4m3 before it is widened.
+int compute_dtype(int32_t dtype) { return dtype == FCK_DTYPE_FP8 ? FCK_DTYPE_BF16 : dtype; }
+
+// The all-fp8 roles of a call (dtype FLOAT8): what the K/V descales do not cover.  `at` may be null.
+int fill_q8(int32_t& q8, float* o_scale, const fck::ScoreMod& mod, const fck_fmha_attrs* at, int32_t dtype)
+{
+    q8 = 0;
+    if (o_scale) *o_scale = 1.f;
+    if (dtype != FCK_DTYPE_FP8) return FCK_OK;
+    // BiasDataType of the fp8 roles is float (fmha_common_jinja.h:157-171): no kernel reads such a bias
+    if (mod.bias_type == FCK_BIAS_ELEMENTWISE) return fail(FCK_ERR_UNSUPPORTED, "an elementwise bias with e4m3 queries has no kernel");
+    const float os = at && at->o_scale != 0.f ? at->o_scale : 1.f;
+    if (!(os > 0.f) || !std::isfinite(os)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_scale must be positive and finite (0: 1)");
+    if (!o_scale && os != 1.f)
+        return fail(FCK_ERR_UNSUPPORTED, "o_scale applies where the output is written: the split-KV partial results are fp32 and "
+                                         "fck_fmha_fwd_splitkv_combine writes e4m3 with scale 1, as the reference's wrapper does");
+    q8 = 1;
+    if (o_scale) *o_scale = os;
     return FCK_OK;
 }
 
@@ -61,13 +85,15 @@ int kernel_dim(int64_t d, int64_t dv)
 
 // fp8 K/V with static per-tensor scales for the prefill entry points (after fill_mod): the K scale multiplies every
 // score, the V scale the output
-int fill_kv8(fck::PrefillArgs& a, const fck_fmha_attrs* at, int64_t d, int64_t dv)
+int fill_kv8(fck::PrefillArgs& a, const fck_fmha_attrs* at, int64_t d, int64_t dv, int32_t dtype)
 {
     a.kv8 = 0;
     a.v_descale = 1.f;
-    if (!at || at->kv_dtype == 0) return FCK_OK;
-    if (at->kv_dtype != FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: only 0 (same as q) and FLOAT8 (1)", at->kv_dtype);
-    const float kd = at->k_descale == 0.f ? 1.f : at->k_descale, vd = at->v_descale == 0.f ? 1.f : at->v_descale;
+    if (int rc = fill_q8(a.q8, &a.o_scale, a.mod, at, dtype)) return rc;
+    const int32_t kvt = at ? at->kv_dtype : 0;
+    if (!a.q8 && kvt == 0) return FCK_OK;  // e4m3 queries: "same as q" is e4m3 too
+    if (kvt != 0 && kvt != FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: only 0 (same as q) and FLOAT8 (1)", kvt);
+    const float kd = !at || at->k_descale == 0.f ? 1.f : at->k_descale, vd = !at || at->v_descale == 0.f ? 1.f : at->v_descale;
     if (!(kd > 0.f) || !std::isfinite(kd) || !(vd > 0.f) || !std::isfinite(vd))
         return fail(FCK_ERR_INVALID_ARGUMENT, "k_descale and v_descale must be positive and finite (0: 1)");
     if (d != dv || d != kernel_dim(d, dv)) return fail(FCK_ERR_UNSUPPORTED, "an fp8 K/V cache needs qk_head_dim = v_head_dim in {64, 128, 256}");
@@ -297,10 +323,12 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
         }
         a.variant = dvar;
     }
-    if (attrs && attrs->kv_dtype != 0) {
+    if (int rc = fill_q8(a.q8, nullptr, a.mod, attrs, dtype)) return rc;
+    if (a.q8 || (attrs && attrs->kv_dtype != 0)) {  // e4m3 queries: "same as q" is e4m3 too
         // fp8 K/V with static per-tensor scales: the K scale multiplies every score, the V scale the output
-        if (attrs->kv_dtype != FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: only 0 (same as q) and FLOAT8 (1)", attrs->kv_dtype);
-        const float kd = attrs->k_descale == 0.f ? 1.f : attrs->k_descale, vd = attrs->v_descale == 0.f ? 1.f : attrs->v_descale;
+        const int32_t kvt = attrs ? attrs->kv_dtype : 0;
+        if (kvt != 0 && kvt != FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "kv_dtype %d: only 0 (same as q) and FLOAT8 (1)", kvt);
+        const float kd = !attrs || attrs->k_descale == 0.f ? 1.f : attrs->k_descale, vd = !attrs || attrs->v_descale == 0.f ? 1.f : attrs->v_descale;
         if (!(kd > 0.f) || !std::isfinite(kd) || !(vd > 0.f) || !std::isfinite(vd))
             return fail(FCK_ERR_INVALID_ARGUMENT, "k_descale and v_descale must be positive and finite (0: 1)");
         if (!aligned16(k) || !aligned16(v)) return fail(FCK_ERR_INVALID_ARGUMENT, "k and v must be 16-byte aligned");
@@ -372,8 +400,8 @@ int fck_fmha_fwd_splitkv_attrs(const void* q, const void* k, const void* v, cons
     a.o_acc = static_cast<float*>(o_acc);
     a.lse_acc = static_cast<float*>(lse_acc);
     int hpw = 1;
-    const hipError_t e = fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream), &hpw);
-    name_decode_kernel(uniform, hpw, a.kv8 != 0, a.mod.active(), d != dv || d != kernel_dim(d, dv), false, a.split_chunk > 0);
+    const hipError_t e = fck::launch_splitkv_decode(a, kernel_dim(d, dv), compute_dtype(dtype), rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream), &hpw);
+    name_decode_kernel(uniform, hpw, a.kv8 != 0, a.mod.active(), d != dv || d != kernel_dim(d, dv), false, a.split_chunk > 0, a.q8 != 0);
     return launch_status(e, "FmhaFwdSplitKV launch");
 }
 
@@ -385,6 +413,7 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
                                int64_t window_left, int64_t window_right, uint32_t mask_type, int32_t dtype, void* stream)
 {
     g_err[0] = 0;
+    if (dtype == FCK_DTYPE_FP8) return fail(FCK_ERR_UNSUPPORTED, "the fused split-KV entry point has no e4m3 kernels");
     // num_splits == 0: the split count comes from the CU count and the longest possible KV length (the capacity of
     // the block table, or seqlen_k), as fck_fmha_num_splits_heuristic gives it
     if (num_splits == 0) {
@@ -428,7 +457,7 @@ int fck_fmha_fwd_splitkv_fused(const void* q, const void* k, const void* v, cons
     a.lse_acc = a.o_acc + part_rows * dv;
     a.o = o;
     int hpw = 1;
-    const hipError_t e = fck::launch_splitkv_decode(a, kernel_dim(d, dv), dtype, rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream), &hpw);
+    const hipError_t e = fck::launch_splitkv_decode(a, kernel_dim(d, dv), compute_dtype(dtype), rows_max, uniform, cu_count(), static_cast<hipStream_t>(stream), &hpw);
     name_decode_kernel(uniform, hpw, false, false, false, true, false);
     return launch_status(e, "FmhaFwdSplitKV (fused) launch");
 }
@@ -477,8 +506,8 @@ int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o
 {
     g_err[0] = 0;
     (void)q_max_seq_len;
-    if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16)
-        return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
+    if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16 && dtype != FCK_DTYPE_FP8)
+        return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT8 (1, e4m3), FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
     if (!lse_acc || !o_acc || !o) return fail(FCK_ERR_INVALID_ARGUMENT, "lse_acc, o_acc and o must not be null");
     if (batch <= 0 || hq <= 0 || seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch, q_num_heads and seqlen_q must be positive");
     if (dv < 8 || dv > 256 || dv % 8) return fail(FCK_ERR_UNSUPPORTED, "v_head_dim %ld: a multiple of 8 in [8, 256]", (long)dv);
@@ -495,6 +524,7 @@ int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o
     a.dv = (int32_t)dv;
     a.num_splits = (int32_t)num_splits;
     a.num_cu = cu_count();
+    a.o_scale = 1.f;  // e4m3 output: the reference's wrapper has no scale argument either (fmha_fwd_split_kv_combine_jinja.h:78-92)
     return launch_status(fck::launch_splitkv_combine(a, dtype, static_cast<hipStream_t>(stream)), "FmhaFwdSplitKVCombine launch");
 }
 
@@ -610,21 +640,22 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t
         if (fast && d <= 128 && q_max_seq_len > 128) {
             a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
             g_kernel = uniform ? "prefill_pp_kernel<uniform_page,padded_head_dim>" : "prefill_pp_kernel<row_lookup,padded_head_dim>";
-            return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+            return launch_status(fck::launch_prefill_pingpong(a, (int)d, compute_dtype(dtype), uniform, static_cast<hipStream_t>(stream)), what);
         }
         a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
         if (fast && d == 256 && uniform) {
             g_kernel = "prefill_dma_kernel<uniform_page,padded_head_dim>";
-            return launch_status(fck::launch_prefill_dma(a, (int)d, dtype, static_cast<hipStream_t>(stream)), what);
+            return launch_status(fck::launch_prefill_dma(a, (int)d, compute_dtype(dtype), static_cast<hipStream_t>(stream)), what);
         }
         g_kernel = uniform ? "prefill_kernel<uniform_page,padded_head_dim>" : "prefill_kernel<row_lookup,padded_head_dim>";
-        return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+        return launch_status(fck::launch_prefill(a, (int)d, compute_dtype(dtype), uniform, static_cast<hipStream_t>(stream)), what);
     }
     if (a.kv8) {
         // an fp8 cache is widened on its way into LDS, which only the register-staged kernel can do
         a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
-        g_kernel = uniform ? "prefill_kernel<uniform_page,kv_fp8>" : "prefill_kernel<row_lookup,kv_fp8>";
-        return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+        g_kernel = a.q8 ? (uniform ? "prefill_kernel<uniform_page,all_fp8>" : "prefill_kernel<row_lookup,all_fp8>")
+                        : (uniform ? "prefill_kernel<uniform_page,kv_fp8>" : "prefill_kernel<row_lookup,kv_fp8>");
+        return launch_status(fck::launch_prefill(a, (int)d, compute_dtype(dtype), uniform, static_cast<hipStream_t>(stream)), what);
     }
     const bool mod = a.mod.active();
     if (mod && a.mod.bias_type == FCK_BIAS_ELEMENTWISE) {
@@ -632,7 +663,7 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t
         // are arithmetic on the score and every kernel applies them
         a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
         g_kernel = uniform ? "prefill_kernel<uniform_page,score_mod>" : "prefill_kernel<row_lookup,score_mod>";
-        return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+        return launch_status(fck::launch_prefill(a, (int)d, compute_dtype(dtype), uniform, static_cast<hipStream_t>(stream)), what);
     }
     if (d <= 128 && q_max_seq_len > 128) {
         a.m_tiles = (int32_t)((q_max_seq_len + 255) / 256);
@@ -641,19 +672,19 @@ static int prefill_common(fck::PrefillArgs& a, int64_t d_qk, int64_t dv, int32_t
                                                 "prefill_pp_kernel<uniform_page,fast_requests,max_in_matrix_phase>"};
         g_kernel = uniform ? (mod ? "prefill_pp_kernel<uniform_page,score_mod>" : variants[a.variant])
                            : (mod ? "prefill_pp_kernel<row_lookup,score_mod>" : "prefill_pp_kernel<row_lookup>");
-        return launch_status(fck::launch_prefill_pingpong(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+        return launch_status(fck::launch_prefill_pingpong(a, (int)d, compute_dtype(dtype), uniform, static_cast<hipStream_t>(stream)), what);
     }
     a.m_tiles = (int32_t)((q_max_seq_len + 127) / 128);
     if (d == 256 && uniform) {
         g_kernel = mod ? "prefill_dma_kernel<uniform_page,score_mod>" : "prefill_dma_kernel<uniform_page>";
-        return launch_status(fck::launch_prefill_dma(a, (int)d, dtype, static_cast<hipStream_t>(stream)), what);
+        return launch_status(fck::launch_prefill_dma(a, (int)d, compute_dtype(dtype), static_cast<hipStream_t>(stream)), what);
     }
     if (mod) {
         g_kernel = uniform ? "prefill_kernel<uniform_page,score_mod>" : "prefill_kernel<row_lookup,score_mod>";
-        return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+        return launch_status(fck::launch_prefill(a, (int)d, compute_dtype(dtype), uniform, static_cast<hipStream_t>(stream)), what);
     }
     g_kernel = uniform ? "prefill_kernel<uniform_page>" : "prefill_kernel<row_lookup>";
-    return launch_status(fck::launch_prefill(a, (int)d, dtype, uniform, static_cast<hipStream_t>(stream)), what);
+    return launch_status(fck::launch_prefill(a, (int)d, compute_dtype(dtype), uniform, static_cast<hipStream_t>(stream)), what);
 }
 
 int fck_fmha_fwd(const void* q, const void* k, const void* v, const void* bias, void* o, const int32_t* seqstart_q,
@@ -692,7 +723,7 @@ int fck_fmha_fwd_attrs(const void* q, const void* k, const void* v, const void* 
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, bias, attrs, scale, mask_type, hq)) return rc;
-    if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
+    if (int rc = fill_kv8(a, attrs, d, dv, dtype)) return rc;
     if (int rc = fill_variant(a, attrs)) return rc;
     a.kv.page_shift = -1;
     a.kv.seqlen_k_ptr = seqlen_k_ptr;  // group mode: logical key counts of padded packed sequences
@@ -747,7 +778,7 @@ int fck_fmha_batch_prefill_attrs(const void* q, const void* k_cache, const void*
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
-    if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
+    if (int rc = fill_kv8(a, attrs, d, dv, dtype)) return rc;
     if (int rc = fill_variant(a, attrs)) return rc;
     a.kv.mode = 3;
     a.kv.kv_indptr = kv_indptr;
@@ -801,7 +832,7 @@ int fck_fmha_fwd_pagedkv_attrs(const void* q, const void* k_cache, const void* v
     a.window_left = window_left;
     a.window_right = window_right;
     if (int rc = fill_mod(a.mod, nullptr, attrs, scale, mask_type, hq)) return rc;
-    if (int rc = fill_kv8(a, attrs, d, dv)) return rc;
+    if (int rc = fill_kv8(a, attrs, d, dv, dtype)) return rc;
     if (int rc = fill_variant(a, attrs)) return rc;
     a.kv.mode = 2;
     a.kv.block_table = block_table;

@@ -51,6 +51,7 @@ struct SplitKvArgs {
     float v_descale;   // factor on the output (1 unless V is quantised)
     int32_t longest_first;  // set by the launcher: workgroups take the sequences in order of decreasing key count
     int32_t d, dv;     // head dims of Q/K and of V/O as stored (multiples of 8); the kernel's D is the next of 64 / 128 / 256
+    int32_t q8;        // with kv8: Q is e4m3 too and P is rounded to e4m3 before the second product (all-fp8 roles)
 };
 
 struct CombineArgs {
@@ -61,6 +62,7 @@ struct CombineArgs {
     int64_t Sq;
     int32_t hq, dv, num_splits;
     int32_t num_cu;  // compute units of the device (decides the workgroup size)
+    float o_scale;   // e4m3 output: O = saturate(o_scale * o)
 };
 
 struct AppendKvArgs {
@@ -101,6 +103,8 @@ struct PrefillArgs {
     int32_t variant;  // tile variant of the ping-pong kernel: 0 / 1 the default schedule, 2..4 see prefill_pingpong.hip
     int32_t kv8;      // K and V are fp8 (e4m3); the K scale is folded into scale_log2 / mod.scale by the caller (4-wave kernel only)
     float v_descale;  // factor on the output (1 unless V is quantised)
+    int32_t q8;       // with kv8: Q and O are e4m3 too, P is rounded to e4m3 before the second product (all-fp8 roles)
+    float o_scale;    // q8: O = saturate(o_scale * o)
 };
 
 // arguments of the paged-cache checker: a block table (block_table != nullptr: seqlen_k, block_table_stride) or a page

@@ -41,6 +41,10 @@ constexpr size_t prefill_lds_bytes()
 // kKv8: K and V are stored as fp8 (e4m3, one byte per element, static per-tensor scales) and widened to T on their way
 // into LDS; a lane then loads 8 bytes where the 16-bit path loads 16.  The K scale arrives folded into the softmax
 // scale, the V scale multiplies the output.  Always together with kMod (the identity when no modifier is set).
+// a.q8 (kKv8 instantiations only): the all-fp8 roles.  Q is e4m3 as well (widened to T like K and V: exact), every
+// probability is rounded to e4m3 before the second product (the row sum keeps the unrounded values), and O is stored as
+// e4m3, saturate(o_scale * o).  The matrix instructions are the 16-bit ones: what the roles save here is memory
+// traffic, not matrix time.
 template <typename T, int D, bool kUniformPage, bool kMod = false, bool kPad = false, bool kKv8 = false>
 __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const PrefillArgs a)
 {
@@ -105,11 +109,26 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
     {
         const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * dq +
                              half * 8;
+        bool q_done = false;
+        if constexpr (kKv8) {
+            if (a.q8) {  // one byte per element
+                const uint8_t* qp8 = reinterpret_cast<const uint8_t*>(a.q) + ((int64_t)(q_row0 + (row_ok ? r : 0)) * a.hq + h) * D + half * 8;
 #pragma unroll
-        for (int t = 0; t < S::KT; ++t) {
-            u32x4_t v = {0u, 0u, 0u, 0u};
-            if (row_ok && (!kPad || t * 16 + half * 8 < dq)) v = ldg16(qp + t * 16);
-            qf[t] = as_vec8<vec8>(v);
+                for (int t = 0; t < S::KT; ++t) {
+                    u32x2_t v = {0u, 0u};
+                    if (row_ok) v = *reinterpret_cast<const u32x2_t*>(qp8 + t * 16);
+                    qf[t] = as_vec8<vec8>(fp8x8_to_t<T>(u32x4_t{v[0], v[1], 0u, 0u}));
+                }
+                q_done = true;
+            }
+        }
+        if (!q_done) {
+#pragma unroll
+            for (int t = 0; t < S::KT; ++t) {
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                if (row_ok && (!kPad || t * 16 + half * 8 < dq)) v = ldg16(qp + t * 16);
+                qf[t] = as_vec8<vec8>(v);
+            }
         }
     }
 
@@ -278,6 +297,18 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
                 psum += p;
             }
         l_run += psum;
+        if constexpr (kKv8) {
+            if (a.q8) {  // 0 <= p <= 2^kLazy = 256 < 448: the conversion never saturates
+#pragma unroll
+                for (int mbk = 0; mbk < 2; ++mbk)
+#pragma unroll
+                    for (int j = 0; j < 16; j += 2) {
+                        const f32x2_t p8 = round_to_fp8(s[mbk][j], s[mbk][j + 1]);
+                        s[mbk][j] = p8[0];
+                        s[mbk][j + 1] = p8[1];
+                    }
+            }
+        }
 
         // ---- O^T += V^T . P^T ---------------------------------------------------------------------------------------
 #pragma unroll
@@ -309,6 +340,20 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void prefill_kernel(const 
     if (row_ok) {
         float inv = (l_run == 0.f) ? 0.f : 1.f / l_run;
         if constexpr (kKv8) inv *= a.v_descale;
+        if constexpr (kKv8) {
+            if (a.q8) {  // four e4m3 bytes per store
+                inv *= a.o_scale;
+                uint8_t* op8 = reinterpret_cast<uint8_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * D;
+#pragma unroll
+                for (int dvb = 0; dvb < S::DVB; ++dvb)
+#pragma unroll
+                    for (int j4 = 0; j4 < 4; ++j4)
+                        *reinterpret_cast<uint32_t*>(op8 + dvb * 32 + j4 * 8 + half * 4) =
+                            pack_fp8x4_sat(oacc[dvb][j4 * 4 + 0] * inv, oacc[dvb][j4 * 4 + 1] * inv, oacc[dvb][j4 * 4 + 2] * inv,
+                                           oacc[dvb][j4 * 4 + 3] * inv);
+                return;
+            }
+        }
         uint16_t* op = reinterpret_cast<uint16_t*>(a.o) + ((int64_t)(q_row0 + r) * a.hq + h) * dvs;
 #pragma unroll
         for (int dvb = 0; dvb < S::DVB; ++dvb)
@@ -330,6 +375,7 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
 {
     const dim3 grid(a.m_tiles, a.hq, a.batch);
     constexpr size_t lds = prefill_lds_bytes<D>();
+    if (a.q8 && !a.kv8) return hipErrorInvalidValue;  // refused by the caller
     if (a.kv8) {  // fp8 cache: the general kernel with the widening load (the caller refuses padded head dims)
         if (a.d != D || a.dv != D) return hipErrorInvalidValue;
         if (uniform) return launch_with_lds<prefill_kernel<T, D, true, true, false, true>>(grid, dim3(256), lds, st, a);

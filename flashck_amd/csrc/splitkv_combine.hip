@@ -9,7 +9,12 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
+#include <type_traits>
+
 namespace fck {
+
+// output type tag: one e4m3 byte per element, O = saturate(a.o_scale * o) (the all-fp8 roles)
+struct FP8Out {};
 
 template <typename T, int DV, int NT = 256>
 __global__ __launch_bounds__(NT) void splitkv_combine_kernel(const CombineArgs a)
@@ -26,10 +31,15 @@ __global__ __launch_bounds__(NT) void splitkv_combine_kernel(const CombineArgs a
     const int64_t w0 = ((b * a.hq + h) * ns) * a.Sq + i;  // split 0; next split is Sq further
 
     const f32x4_t acc = combine_splits<DV>(a.lse_acc, a.o_acc, w0, a.Sq, ns, c, a.dv);
-    u32x2_t out;
-    out[0] = T::pack2(acc[0], acc[1]);
-    out[1] = T::pack2(acc[2], acc[3]);
-    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.o) + (row * a.hq + h) * a.dv + c) = out;
+    if constexpr (std::is_same<T, FP8Out>::value) {
+        *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(a.o) + (row * a.hq + h) * a.dv + c) =
+            pack_fp8x4_sat(acc[0] * a.o_scale, acc[1] * a.o_scale, acc[2] * a.o_scale, acc[3] * a.o_scale);
+    } else {
+        u32x2_t out;
+        out[0] = T::pack2(acc[0], acc[1]);
+        out[1] = T::pack2(acc[2], acc[3]);
+        *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.o) + (row * a.hq + h) * a.dv + c) = out;
+    }
 }
 
 template <typename T, int DV>
@@ -57,6 +67,7 @@ static hipError_t launch_t(const CombineArgs& a, hipStream_t st)
 
 hipError_t launch_splitkv_combine(const CombineArgs& a, int dtype, hipStream_t st)
 {
+    if (dtype == 1) return launch_t<FP8Out>(a, st);
     return dtype == 4 ? launch_t<BF16>(a, st) : launch_t<FP16>(a, st);
 }
 

@@ -61,6 +61,9 @@ __device__ __forceinline__ int v_swizzle(int key)
 
 // kKv8: K and V are stored as fp8 (e4m3, one byte per element) and widened to T on their way into LDS; everything after
 // the staging tile is the 16-bit path.  A lane then loads 8 bytes where the 16-bit path loads 16.
+// a.q8 (instantiations with kMod and kKv8 only): the all-fp8 roles.  Q is e4m3 as well (widened to T like K and V: exact)
+// and every probability is rounded to e4m3 before the second product (the row sum keeps the unrounded values).  The
+// partial results stay fp32; the e4m3 output is written by the combine kernel.
 // kPad: the stored head dims (a.d for Q/K, a.dv for V and the output; multiples of 8) are smaller than D: rows are
 // a.d / a.dv elements apart, and the 16-byte pieces past a row's end are zeros instead of loads (a zero column of Q and K
 // adds nothing to a score, a zero column of V gives an output column that is not stored).
@@ -193,6 +196,18 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
                 const int64_t off = ((int64_t)(q_row0 + row_i[mb]) * a.hq + (hkv0 + hl) * g + row_hl[mb]) * dq + kg * 8;
+                if constexpr (kMod && kKv8) {
+                    if (a.q8) {  // one byte per element
+                        const uint8_t* qp8 = reinterpret_cast<const uint8_t*>(a.q) + off;
+#pragma unroll
+                        for (int t = 0; t < S::KT; ++t) {
+                            u32x2_t v = {0u, 0u};
+                            if (row_ok[mb]) v = *reinterpret_cast<const u32x2_t*>(qp8 + t * 32);
+                            qf[hl][mb][t] = as_vec8<vec8>(fp8x8_to_t<T>(u32x4_t{v[0], v[1], 0u, 0u}));
+                        }
+                        continue;
+                    }
+                }
 #pragma unroll
                 for (int t = 0; t < S::KT; ++t) {
                     u32x4_t v = {0u, 0u, 0u, 0u};
@@ -407,6 +422,16 @@ __global__ __launch_bounds__(NW * 64) void splitkv_decode_kernel(const SplitKvAr
                     psum += p[e];
                 }
                 l_run[hl][mb] = l_run[hl][mb] * alpha + psum;
+                if constexpr (kMod && kKv8) {
+                    if (a.q8) {  // 0 <= p <= 1: the conversion never saturates
+#pragma unroll
+                        for (int e = 0; e < 4 * S::NBK; e += 2) {
+                            const f32x2_t p8 = round_to_fp8(p[e], p[e + 1]);
+                            p[e] = p8[0];
+                            p[e + 1] = p8[1];
+                        }
+                    }
+                }
 #pragma unroll
                 for (int db = 0; db < S::DB; ++db) oacc[hl][mb][db] *= alpha;
 #pragma unroll
@@ -590,6 +615,7 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
     const dim3 grid((unsigned)((int64_t)(a.hk / HG) * a.num_splits * a.m_tiles * a.batch));
     const dim3 block(NW * 64);
     constexpr size_t lds = decode_lds_bytes<D, NW, HG>();
+    if (a.q8 && (!a.kv8 || a.tickets || a.d != D || a.dv != D)) return hipErrorInvalidValue;  // refused by the caller
     if constexpr (HG == 1) {
         if (a.d != D || a.dv != D) {  // padded head dims: the general kernel (modifiers on, identity when there are none)
             if (a.kv8 || a.tickets) return hipErrorInvalidValue;  // refused by the caller
@@ -597,7 +623,7 @@ static hipError_t launch_cfg(const SplitKvArgs& a, bool uniform, hipStream_t st)
             return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true, false, true>>(grid, block, lds, st, a);
         }
     }
-    if (a.mod.active()) {
+    if (a.mod.active() || a.q8) {  // q8 (all-fp8 roles) lives in the general fp8 kernels only
         if (a.kv8) {
             if (uniform) return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, true, true, true>>(grid, block, lds, st, a);
             return launch_with_lds<splitkv_decode_kernel<T, D, NW, MB, HG, false, true, true>>(grid, block, lds, st, a);

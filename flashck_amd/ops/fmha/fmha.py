@@ -32,7 +32,9 @@ __all__ = [
 MASK_NONE, MASK_TOP_LEFT, MASK_BOTTOM_RIGHT, MASK_GENERIC = 0, 1, 2, 3
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALF_ROTATED = 0, 1, 2
 
-_DTYPE_ID = {torch.float16: 3, torch.bfloat16: 4}  # flashck::DataType, core/utils/dtype.h:16-28
+# flashck::DataType, core/utils/dtype.h:16-28.  float8_e4m3fn queries select the all-fp8 roles (Q, K, V, P and O in e4m3,
+# FmhaFwdTypeConfig<fp8_t>, core/module/kernels/attention_kernels/fmha_common_jinja.h:157-171).
+_DTYPE_ID = {torch.float8_e4m3fn: 1, torch.float16: 3, torch.bfloat16: 4}
 
 
 # Host-side tests of the validation code switch this off (and replace _call); nothing else may.
@@ -41,7 +43,7 @@ _REQUIRE_GPU_TENSORS = True
 
 def _dtype_id(t: torch.Tensor) -> int:
     if t.dtype not in _DTYPE_ID:
-        raise TypeError(f"FMHA supports torch.float16 and torch.bfloat16, got {t.dtype}")
+        raise TypeError(f"FMHA supports torch.float16, torch.bfloat16 and torch.float8_e4m3fn, got {t.dtype}")
     return _DTYPE_ID[t.dtype]
 
 
@@ -123,9 +125,11 @@ def _window(window):
 
 
 def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols, kv_fp8=False, k_descale=1.0, v_descale=1.0,
-           decode_variant=0, prefill_variant=0, max_seqlen_k=0):
+           decode_variant=0, prefill_variant=0, max_seqlen_k=0, o_scale=1.0):
     """fck_fmha_attrs for a call, or None when no score modifier is asked for.
 
+    o_scale (float8_e4m3fn queries on the dense / paged / page-list prefill calls): the output is
+    saturate(o_scale * o) in e4m3.
     bias (elementwise, BiasEnum ELEMENTWISE_BIAS): q's dtype, last dim contiguous; batch mode [1|B, 1|Hq, sq, >= sk],
     group mode [1|Hq, total_q, >= max sk]; size-1 dims are shared (the reference's rank 0 / 1 / 2).
     alibi_slopes (ALIBI): fp32 [Hq] or [B, Hq].  logits_soft_cap > 0: s = cap * tanh(scale * qk / cap).
@@ -152,6 +156,9 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
         if not (float(k_descale) > 0.0 and float(v_descale) > 0.0 and math.isfinite(k_descale) and math.isfinite(v_descale)):
             raise ValueError("k_descale and v_descale must be positive and finite")
         a.kv_dtype, a.k_descale, a.v_descale = 1, float(k_descale), float(v_descale)  # flashck::DataType FLOAT8
+    if not (float(o_scale) > 0.0 and math.isfinite(o_scale)):
+        raise ValueError("o_scale must be positive and finite")
+    a.o_scale = float(o_scale)
     Hq = q.shape[-2]
     if bias is not None:
         if not isinstance(bias, torch.Tensor):
@@ -244,9 +251,10 @@ def splitkv_workspace(shape_batch, q_num_heads, shape_seqlen_q, v_head_dim, num_
 
 def fmha_fwd(q, k, v, scale: float = 0.0, mask_type: int = MASK_NONE, window: Tuple[int, int] = (-1, -1),
              seqlen_k: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, *, bias=None, alibi_slopes=None,
-             logits_soft_cap: float = 0.0) -> torch.Tensor:
+             logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0, o_scale: float = 1.0) -> torch.Tensor:
     """Dense attention, batch mode: q [B,sq,Hq,D], k/v [B,sk,Hk,D] -> o [B,sq,Hq,D].
-    bias / alibi_slopes / logits_soft_cap: see _attrs."""
+    bias / alibi_slopes / logits_soft_cap: see _attrs.  float8_e4m3fn tensors: the all-fp8 roles, with k = k_descale *
+    stored, v = v_descale * stored, o = saturate(o_scale * result)."""
     _check_tensor("q", q, ndim=4)
     _check_tensor("k", k, dtype=q.dtype, ndim=4)
     _check_tensor("v", v, dtype=q.dtype, ndim=4)
@@ -262,7 +270,8 @@ def fmha_fwd(q, k, v, scale: float = 0.0, mask_type: int = MASK_NONE, window: Tu
     sk, Hk, Dv = k.shape[1], k.shape[2], v.shape[3]
     o = _out("out", out, (B, sq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
-    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, False, B, sq, sk)
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, False, B, sq, sk, q.dtype == torch.float8_e4m3fn, k_descale, v_descale,
+                      o_scale=o_scale)
     if at is None:
         _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), None, None, _ptr(seqlen_k), B, sq, sk, Hq, Hk, D, Dv,
               sq, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
@@ -275,9 +284,9 @@ def fmha_fwd(q, k, v, scale: float = 0.0, mask_type: int = MASK_NONE, window: Tu
 
 def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scale: float = 0.0,
                     mask_type: int = MASK_NONE, window=(-1, -1), seqlen_k=None, out=None, *, bias=None, alibi_slopes=None,
-                    logits_soft_cap: float = 0.0) -> torch.Tensor:
+                    logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0, o_scale: float = 1.0) -> torch.Tensor:
     """Dense attention, group mode: q [total_q,Hq,D], k/v [total_k,Hk,D] packed by cu_seqlens.
-    bias / alibi_slopes / logits_soft_cap: see _attrs.
+    bias / alibi_slopes / logits_soft_cap: see _attrs; float8_e4m3fn tensors and their scales: see fmha_fwd.
 
     seqlen_k (int32 [B], optional): logical key counts when the packed K/V slots hold padding behind the keys."""
     _check_tensor("q", q, ndim=3)
@@ -296,7 +305,8 @@ def fmha_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, scal
     Hk, Dv = k.shape[1], v.shape[2]
     o = _out("out", out, (tq, Hq, Dv), q.dtype, q)
     wl, wr = _window(window)
-    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1)
+    at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1, q.dtype == torch.float8_e4m3fn, k_descale, v_descale,
+                      o_scale=o_scale)
     if at is None:
         _call("fck_fmha_fwd", _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), _ptr(seqlen_k), B, tq,
               k.shape[0], Hq, Hk, D, Dv, max_seqlen_q, _scale(scale, D), wl, wr, mask_type, _dtype_id(q), _stream())
@@ -448,7 +458,7 @@ def fmha_fwd_splitkv_fused(q, k, v, num_splits: int = 0, *, seqlen_k=None, block
 def fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype, cu_seqlens_q=None, max_seqlen_q: int = 0, out=None) -> torch.Tensor:
     """LSE combine of split-KV partials -> o [B,sq,Hq,Dv] (or [total_q,Hq,Dv] in group mode)."""
     if dtype not in _DTYPE_ID:
-        raise TypeError(f"FMHA supports torch.float16 and torch.bfloat16, got {dtype}")
+        raise TypeError(f"FMHA supports torch.float16, torch.bfloat16 and torch.float8_e4m3fn, got {dtype}")
     _check_tensor("lse_acc", lse_acc, dtype=torch.float32, ndim=4)
     _check_tensor("o_acc", o_acc, dtype=torch.float32, ndim=5)
     _check_tensor("cu_seqlens_q", cu_seqlens_q, dtype=torch.int32, optional=True)
@@ -574,10 +584,11 @@ def tune_prefill_variant(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_i
 def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_indices, kv_last_page_lens=None, *,
                        max_seqlen_q: int, scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0),
                        out=None, bias=None, alibi_slopes=None, logits_soft_cap: float = 0.0, k_descale: float = 1.0,
-                       v_descale: float = 1.0, prefill_variant: int = 0) -> torch.Tensor:
+                       v_descale: float = 1.0, prefill_variant: int = 0, o_scale: float = 1.0) -> torch.Tensor:
     """Varlen prefill over a page list: q [total_q,Hq,D]; sequence b owns pages
     kv_page_indices[kv_indptr[b]:kv_indptr[b+1]] of the cache [num_pages, page_size, Hk, D].  The caches may be
-    torch.float8_e4m3fn with the static scales k_descale / v_descale (value = descale * stored)."""
+    torch.float8_e4m3fn with the static scales k_descale / v_descale (value = descale * stored); with float8_e4m3fn
+    queries as well (the all-fp8 roles) the output is float8_e4m3fn, saturate(o_scale * result)."""
     _check_tensor("q", q, ndim=3)
     kv_fp8 = isinstance(k_cache, torch.Tensor) and k_cache.dtype == torch.float8_e4m3fn
     _check_tensor("k_cache", k_cache, dtype=torch.float8_e4m3fn if kv_fp8 else q.dtype, ndim=4)
@@ -602,7 +613,7 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
         prefill_variant = _usable_prefill_variant(tuning.choose_prefill_variant(tuning.prefill_problem(
             Hq, Hk, D, max_seqlen_q, tq, page, "fp16" if q.dtype == torch.float16 else "bf16", mask_type)), D, Dv, max_seqlen_q, page)
     at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, True, B, tq, 1, kv_fp8, k_descale, v_descale,
-                      prefill_variant=prefill_variant)
+                      prefill_variant=prefill_variant, o_scale=o_scale)
     if at is None:
         _call("fck_fmha_batch_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(kv_indptr),
               _ptr(kv_page_indices), _ptr(kv_last_page_lens), num_pages, page, B, Hq, Hk, D, Dv, max_seqlen_q,
@@ -618,9 +629,10 @@ def fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_ind
 def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q=None, max_seqlen_q: int = 0,
                      scale: float = 0.0, mask_type: int = MASK_BOTTOM_RIGHT, window=(-1, 0), out=None, bias=None,
                      alibi_slopes=None, logits_soft_cap: float = 0.0, k_descale: float = 1.0, v_descale: float = 1.0,
-                     prefill_variant: int = 0) -> torch.Tensor:
+                     prefill_variant: int = 0, o_scale: float = 1.0) -> torch.Tensor:
     """Prefill over a block table (no splits): q [B,sq,Hq,D] or packed [total_q,Hq,D].  The caches may be
-    torch.float8_e4m3fn with the static scales k_descale / v_descale (value = descale * stored)."""
+    torch.float8_e4m3fn with the static scales k_descale / v_descale (value = descale * stored); float8_e4m3fn queries
+    and o_scale: see fmha_batch_prefill."""
     group = cu_seqlens_q is not None
     _check_tensor("q", q, ndim=3 if group else 4)
     kv_fp8 = isinstance(k_cache, torch.Tensor) and k_cache.dtype == torch.float8_e4m3fn
@@ -644,7 +656,7 @@ def fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_q
     wl, wr = _window(window)
     _debug_validate(seqlen_k=seqlen_k, block_table=block_table, num_total_pages=k_cache.shape[0], page_size=page)
     at, keep = _attrs(q, bias, alibi_slopes, logits_soft_cap, group, B, q.shape[0] if group else sq, 1, kv_fp8, k_descale, v_descale,
-                      prefill_variant=prefill_variant)
+                      prefill_variant=prefill_variant, o_scale=o_scale)
     if at is None:
         _call("fck_fmha_fwd_pagedkv", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(o), _ptr(cu_seqlens_q), _ptr(seqlen_k),
               _ptr(block_table), block_table.shape[1], page, B, sq, Hq, Hk, D, Dv, max_seqlen_q or sq, _scale(scale, D), wl, wr,

@@ -37,7 +37,16 @@ extern "C" {
 #define FCK_EXPORT __attribute__((visibility("default")))
 
 /* flashck::DataType, core/utils/dtype.h:16-28 */
-#define FCK_DTYPE_FP8 1 /* e4m3 (OCP, as ck_tile::fp8_t on gfx950); accepted as fck_fmha_attrs.kv_dtype only */
+/* e4m3 (OCP, as ck_tile::fp8_t on gfx950).  As fck_fmha_attrs.kv_dtype: an fp8 K/V cache under 16-bit queries.  As the
+ * `dtype` of fck_fmha_fwd / _pagedkv / _batch_prefill / _splitkv (+ _attrs) and _splitkv_combine: the all-fp8 roles of
+ * FmhaFwdTypeConfig<fp8_t> (core/module/kernels/attention_kernels/fmha_common_jinja.h:157-171): Q, K, V and O are one
+ * e4m3 byte per element, P is rounded to e4m3 before the second product (scale_p = 1, as the reference passes it:
+ * fmha_fwd_jinja.h:327), LSE and the split-KV partial results stay fp32.  k = k_descale * stored, v = v_descale * stored
+ * as for an fp8 cache (a query scale belongs into `scale`); O = saturate(o_scale * o).  Needs qk_head_dim = v_head_dim in
+ * {64, 128, 256}; no elementwise bias (its type would be fp32); not on fck_fmha_fwd_splitkv_fused / _appendkv.  The
+ * products run on the bf16 matrix instructions (every e4m3 value is a bf16 value): the roles halve the memory traffic,
+ * they do not double the matrix rate. */
+#define FCK_DTYPE_FP8 1
 #define FCK_DTYPE_FP16 3
 #define FCK_DTYPE_BF16 4
 
@@ -115,6 +124,9 @@ typedef struct fck_fmha_attrs {
     /* decode_variant 3 / 4: upper bound of the key counts of the batch (0 or anything above the block table's capacity:
      * that capacity).  A bound below a real key count costs balance, not correctness. */
     int64_t max_seqlen_k;
+    /* dtype FCK_DTYPE_FP8 on fck_fmha_fwd / _pagedkv / _batch_prefill: the output is saturate(o_scale * o) in e4m3
+     * (ck_tile's scale_o; the reference passes 1).  0 means 1.  The split-KV pair writes with scale 1. */
+    float o_scale;
 } fck_fmha_attrs;
 
 #define FCK_OK 0

@@ -145,13 +145,25 @@ uint8_t fck_orc_f32_to_fp8(float f)
 
 static inline float ld(const void* base, int64_t idx, int dtype)
 {
+    if (dtype == FCK_ORC_FP8) return fck_orc_fp8_to_f32(((const uint8_t*)base)[idx]);
     uint16_t x = ((const uint16_t*)base)[idx];
     return dtype == FCK_ORC_BF16 ? bf16_to_f32(x) : fp16_to_f32(x);
 }
 static inline uint16_t cvt(float f, int dtype) { return dtype == FCK_ORC_BF16 ? f32_to_bf16(f) : f32_to_fp16(f); }
 static inline float rnd(float f, int dtype)
 {
+    if (dtype == FCK_ORC_FP8) return fck_orc_fp8_to_f32(fck_orc_f32_to_fp8(f));
     return dtype == FCK_ORC_BF16 ? bf16_to_f32(f32_to_bf16(f)) : fp16_to_f32(f32_to_fp16(f));
+}
+/* element idx of an output tensor.  fp8 outputs: o_acc_element_func = saturates<fp8_t> after scales{scale_o}
+   (ck_tile/ops/fmha/kernel/fmha_fwd_kernel.hpp:1530-1538); the reference passes scale_o = 1
+   (core/module/kernels/attention_kernels/fmha_fwd/fmha_fwd_jinja.h:327-328). */
+static inline void st(void* base, int64_t idx, float f, int dtype, float o_scale)
+{
+    if (dtype == FCK_ORC_FP8)
+        ((uint8_t*)base)[idx] = fck_orc_f32_to_fp8(f * (o_scale != 0.f ? o_scale : 1.f));
+    else
+        ((uint16_t*)base)[idx] = cvt(f, dtype);
 }
 
 int fck_orc_num_threads(void)
@@ -270,7 +282,7 @@ static void attend_row(const fck_orc_problem* p, const void* q, const void* k, c
     mask_coords(p->mask_type, p->window_left, p->window_right, sq_b, sk_b, &y, &x);
     for (int t = 0; t < d; ++t) sc->qf[t] = ld(q, (qrow * p->hq + h) * d + t, dt);
 
-    const int kv8 = p->kv_dtype == FCK_ORC_FP8;
+    const int kv8 = p->kv_dtype == FCK_ORC_FP8 || dt == FCK_ORC_FP8; /* all-fp8 roles: Q, K, V, P and O are e4m3 */
     const float kd = (kv8 && p->k_descale != 0.f) ? p->k_descale : 1.f, vd = (kv8 && p->v_descale != 0.f) ? p->v_descale : 1.f;
     /* bias row of (b, h, i) / ALiBi slope of (b, h) */
     int64_t bias_row = 0;
@@ -346,7 +358,8 @@ static int max_sk(const fck_orc_problem* p)
 
 static int check(const fck_orc_problem* p)
 {
-    if (p->dtype != FCK_ORC_BF16 && p->dtype != FCK_ORC_FP16) return -1;
+    if (p->dtype != FCK_ORC_BF16 && p->dtype != FCK_ORC_FP16 && p->dtype != FCK_ORC_FP8) return -1;
+    if (p->dtype == FCK_ORC_FP8 && p->bias_type == 1) return -3; /* BiasDataType of the fp8 roles is float: not restated */
     if (p->hk <= 0 || p->hq % p->hk) return -2;
     return 0;
 }
@@ -380,8 +393,8 @@ int fck_orc_fmha_fwd(const fck_orc_problem* p, const void* q, const void* k, con
                 const int h = (int)(t / sq_b), i = (int)(t % sq_b);
                 float l;
                 attend_row(p, q, k, v, b, row0 + i, h, rows, 0, sk_b, i, sq_b, sk_b, &sc, &l);
-                uint16_t* orow = (uint16_t*)o + ((row0 + i) * p->hq + h) * p->dv;
-                for (int c = 0; c < p->dv; ++c) orow[c] = cvt(sc.of[c], p->dtype);
+                const int64_t orow = ((row0 + i) * p->hq + h) * p->dv;
+                for (int c = 0; c < p->dv; ++c) st(o, orow + c, sc.of[c], p->dtype, p->o_scale);
                 if (lse) {
                     if (p->seqstart_q)
                         lse[(int64_t)h * tq + row0 + i] = l;
@@ -456,9 +469,9 @@ int fck_orc_fmha_splitkv(const fck_orc_problem* p, const void* q, const void* k,
    m = max_s lse_s; sum = sum_s exp(lse_s - m) (0 when m = -inf); LSE = ln(sum) + m (-inf when sum = 0);
    w_s = exp(lse_s - LSE) (0 when LSE = -inf); O = sum_s w_s * O_s, stored in the data type. */
 int fck_orc_splitkv_combine(const float* lse_acc, const float* o_acc, void* o, float* lse, const int32_t* seqstart_q,
-                            int batch, int sq, int hq, int dv, int num_splits, int dtype)
+                            int batch, int sq, int hq, int dv, int num_splits, int dtype, float o_scale)
 {
-    if (dtype != FCK_ORC_BF16 && dtype != FCK_ORC_FP16) return -1;
+    if (dtype != FCK_ORC_BF16 && dtype != FCK_ORC_FP16 && dtype != FCK_ORC_FP8) return -1;
     const int group = seqstart_q != 0;
     const int64_t Sq = group ? seqstart_q[batch] : sq;
     const int Bs = group ? 1 : batch;
@@ -476,14 +489,14 @@ int fck_orc_splitkv_combine(const float* lse_acc, const float* o_acc, void* o, f
                 if (!(isinf(m) && m < 0))
                     for (int s = 0; s < num_splits; ++s) sum += expf(lse_acc[w0 + s * Sq] - m);
                 float L = (sum == 0.f) ? -INFINITY : logf(sum) + m;
-                uint16_t* orow = (uint16_t*)o + (((int64_t)b * Sq + i) * hq + h) * dv;
+                const int64_t orow = (((int64_t)b * Sq + i) * hq + h) * dv;
                 for (int c = 0; c < dv; ++c) {
                     float acc = 0.f;
                     for (int s = 0; s < num_splits; ++s) {
                         float w = (isinf(L) && L < 0) ? 0.f : expf(lse_acc[w0 + s * Sq] - L);
                         acc += w * o_acc[(w0 + s * Sq) * dv + c];
                     }
-                    orow[c] = cvt(acc, dtype);
+                    st(o, orow + c, acc, dtype, o_scale);
                 }
                 if (lse) lse[((int64_t)b * hq + h) * Sq + i] = L;
             }

@@ -76,6 +76,11 @@ typedef struct {
        is_static_quant: core/profiling/attention/fmha_fwd_split_kv/fmha_fwd_split_kv_problem.h:79. */
     int32_t kv_dtype;
     float k_descale, v_descale;
+    /* dtype FCK_ORC_FP8: the all-fp8 roles of FmhaFwdTypeConfig<fp8_t> (fmha_common_jinja.h:157-171): Q, K, V, P and O are
+       e4m3 (K/V as with kv_dtype FCK_ORC_FP8, the descales apply).  P is cast to e4m3 before the second product
+       (p_compute_element_func = scales{scale_p}, scale_p = 1 in the reference) and O = saturate(o_scale * o) (0 means 1;
+       the reference passes scale_o = 1).  ck_tile/ops/fmha/kernel/fmha_fwd_kernel.hpp:1529-1553. */
+    float o_scale;
 } fck_orc_problem;
 
 /* 1 when key j is visible to query i. */
@@ -91,7 +96,7 @@ int fck_orc_fmha_splitkv(const fck_orc_problem* p, const void* q, const void* k,
 
 int fck_orc_splitkv_combine(const float* lse_acc, const float* o_acc, void* o, float* lse,
                             const int32_t* seqstart_q, int batch, int sq, int hq, int dv,
-                            int num_splits, int dtype);
+                            int num_splits, int dtype, float o_scale);
 
 /* x: [rows, heads, d] in place; row r uses table row pos[r]; cos/sin: [*, rotary_dim/2] in the data dtype. */
 int fck_orc_rope(void* x, int rows, int heads, int d, const int32_t* pos, const void* cos_tab,

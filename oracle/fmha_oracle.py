@@ -46,6 +46,7 @@ class _Problem(ctypes.Structure):
         ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64),
         ("logits_soft_cap", ctypes.c_float),
         ("kv_dtype", ctypes.c_int32), ("k_descale", ctypes.c_float), ("v_descale", ctypes.c_float),
+        ("o_scale", ctypes.c_float),
     ]
 
 
@@ -66,7 +67,7 @@ def lib():
                                          ctypes.c_int, ctypes.c_int]
         _lib.fck_orc_fmha_fwd.argtypes = [ctypes.c_void_p] * 6
         _lib.fck_orc_fmha_splitkv.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
-        _lib.fck_orc_splitkv_combine.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6
+        _lib.fck_orc_splitkv_combine.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_float]
         _lib.fck_orc_rope.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                       ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _lib.fck_orc_appendkv.argtypes = ([ctypes.c_void_p] * 9 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int,
@@ -93,7 +94,9 @@ def dtype_id(t):
         return BF16
     if t == torch.float16:
         return FP16
-    raise TypeError(f"oracle supports fp16/bf16 only, got {t}")
+    if t == torch.float8_e4m3fn:   # the all-fp8 roles: Q, K, V, P and O
+        return FP8
+    raise TypeError(f"oracle supports fp16 / bf16 / fp8 (e4m3) only, got {t}")
 
 
 def _ptr(t):
@@ -113,7 +116,7 @@ def _i32(t):
 def _problem(q, k, v, *, seqstart_q=None, seqstart_k=None, seqlen_k=None, block_table=None, page_size=0,
              kv_indptr=None, kv_page_indices=None, kv_last_page_lens=None, cache_batch_idx=None, scale=None,
              mask_type=NO_MASK, window=(-1, -1), batch=None, bias=None, alibi_slopes=None, logits_soft_cap=0.0,
-             k_descale=1.0, v_descale=1.0):
+             k_descale=1.0, v_descale=1.0, o_scale=1.0):
     """bias: data dtype, [1|B, 1|Hq, sq, sk] (batch mode) or [1|Hq, total_q, max_sk] (group mode), last dim contiguous;
     alibi_slopes: fp32 [Hq] or [B, Hq]; logits_soft_cap > 0: s = cap * tanh(scale * qk / cap)."""
     p = _Problem()
@@ -156,6 +159,9 @@ def _problem(q, k, v, *, seqstart_q=None, seqstart_k=None, seqlen_k=None, block_
     if k.dtype == torch.float8_e4m3fn:   # fp8 K/V with static scales
         assert v.dtype == torch.float8_e4m3fn
         p.kv_dtype, p.k_descale, p.v_descale = FP8, float(k_descale), float(v_descale)
+    if q.dtype == torch.float8_e4m3fn:   # fp8 Q, P and O as well: O = saturate(o_scale * o)
+        assert k.dtype == torch.float8_e4m3fn, "fp8 queries come with an fp8 K/V"
+        p.o_scale = float(o_scale)
     assert bias is None or alibi_slopes is None, "one bias kind at a time"
     if bias is not None:
         assert bias.dtype == q.dtype and bias.device.type == "cpu" and bias.stride(-1) == 1
@@ -205,7 +211,7 @@ def fmha_splitkv(q, k, v, num_splits, **kw):
     return o_acc, lse_acc
 
 
-def splitkv_combine(lse_acc, o_acc, dtype, seqstart_q=None, batch=None, return_lse=False):
+def splitkv_combine(lse_acc, o_acc, dtype, seqstart_q=None, batch=None, return_lse=False, o_scale=1.0):
     bs, hq, ns, sq, dv = o_acc.shape
     if seqstart_q is not None:
         o = torch.empty(sq, hq, dv, dtype=dtype)
@@ -215,7 +221,7 @@ def splitkv_combine(lse_acc, o_acc, dtype, seqstart_q=None, batch=None, return_l
         nb = bs
     lse = torch.empty(bs, hq, sq, dtype=torch.float32) if return_lse else None
     rc = lib().fck_orc_splitkv_combine(_ptr(lse_acc), _ptr(o_acc), _ptr(o), _ptr(lse), _i32(seqstart_q), nb, sq, hq, dv,
-                                       ns, dtype_id(dtype))
+                                       ns, dtype_id(dtype), float(o_scale))
     assert rc == 0, rc
     return (o, lse) if return_lse else o
 

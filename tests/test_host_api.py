@@ -193,3 +193,48 @@ def test_validate_paged_arguments_are_checked_before_any_launch():
     assert rc == -1 and b"seqlen_k" in lib.fck_last_error()
     rc = lib.fck_fmha_validate_paged(p, p, 2, None, None, None, 1, 4, 16, None, None)       # no counters
     assert rc == -1 and b"error_counts" in lib.fck_last_error()
+
+
+def test_fp8_roles_are_validated_before_any_launch():
+    """dtype FLOAT8 (1): what the all-fp8 roles do not cover is refused with FCK_ERR_UNSUPPORTED, bad scales with
+    FCK_ERR_INVALID_ARGUMENT; no GPU is needed to get that far."""
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    FP8 = 1
+    # stored head dims other than 64 / 128 / 256, or unequal
+    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 96, 96, 8, 0.125, -1, -1, 0, FP8, None)
+    assert rc == -2 and b"e4m3" in lib.fck_last_error()
+    rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 128, 64, 8, 0.125, -1, -1, 0, FP8, None)
+    assert rc == -2 and b"e4m3" in lib.fck_last_error()
+    # an elementwise bias (it would be fp32 for these roles)
+    at = _lib.Attrs()
+    at.size = ctypes.sizeof(_lib.Attrs)
+    at.bias_type, at.bias, at.bias_row_stride, at.bias_cols = 1, p.value, 8, 8
+    rc = lib.fck_fmha_fwd_attrs(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, FP8, ctypes.byref(at), None)
+    assert rc == -2 and b"bias" in lib.fck_last_error()
+    # scales
+    at = _lib.Attrs()
+    at.size = ctypes.sizeof(_lib.Attrs)
+    at.o_scale = -1.0
+    rc = lib.fck_fmha_fwd_attrs(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, FP8, ctypes.byref(at), None)
+    assert rc == -1 and b"o_scale" in lib.fck_last_error()
+    at.o_scale, at.kv_dtype = 0.0, 4
+    rc = lib.fck_fmha_fwd_attrs(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, FP8, ctypes.byref(at), None)
+    assert rc == -2 and b"kv_dtype" in lib.fck_last_error()
+    # the split-KV partial results are fp32: an output scale has nowhere to go
+    at = _lib.Attrs()
+    at.size = ctypes.sizeof(_lib.Attrs)
+    at.o_scale = 2.0
+    rc = lib.fck_fmha_fwd_splitkv_attrs(p, p, p, None, p, p, None, None, None, None, None, 1, 1, 8, 2, 2, 64, 64, 1, 2, 0, 0, 0.125, -1, -1,
+                                        0, FP8, ctypes.byref(at), None)
+    assert rc == -2 and b"o_scale" in lib.fck_last_error()
+    # the one-launch entry point and appendKV have no e4m3 kernels
+    rc = lib.fck_fmha_fwd_splitkv_fused(p, p, p, None, p, None, None, None, None, None, 1, 1, 8, 2, 2, 64, 64, 1, 2, 0, 0, 0.125, -1, -1, 0,
+                                        FP8, None)
+    assert rc == -2 and b"e4m3" in lib.fck_last_error()
+    rc = lib.fck_fmha_fwd_appendkv(None, p, p, p, p, p, None, 1, None, None, 0, 0, 0, None, 0, 0, None, 0, 1, 2, 2, 64, 64, FP8, None)
+    assert rc == -2
+    # an unknown dtype still names the ones there are
+    rc = lib.fck_fmha_fwd_splitkv_combine(p, p, p, None, 1, 1, 2, 64, 1, 2, 9, None)
+    assert rc == -2 and b"FLOAT8" in lib.fck_last_error()
