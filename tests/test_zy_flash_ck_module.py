@@ -81,3 +81,25 @@ def test_batch_prefill_and_pagedkv(fck, orc):
     sl = torch.tensor(lens, dtype=torch.int32)
     o2 = fck.fmha_fwd_pagedkv(a[0], a[1], a[2], dev(sl), dev(bt), cu_seqlens_q=a[3], max_seqlen_q=w["max_seqlen_q"], scale=w["scale"])
     assert_close(o2, ro, 2e-2, "fmha_fwd_pagedkv")
+
+
+def test_e4m3_tensors_take_the_all_fp8_roles(fck):
+    """float8_e4m3fn q / k / v through the compiled module: the two-key closed form (88 with the cast of P, 96 without;
+    see test_zx_fp8_roles) on the dense call and on split-KV + combine."""
+    f8 = torch.float8_e4m3fn
+    q = torch.zeros(1, 1, 1, 64)
+    q[..., 0] = 1.0
+    k = torch.zeros(1, 2, 1, 64)
+    k[0, 1, 0, 0] = -1.25
+    v = torch.zeros(1, 2, 1, 64)
+    v[0, 1] = 416.0
+    q, k, v = dev(q.to(f8)), dev(k.to(f8)), dev(v.to(f8))
+    o = fck.fmha_fwd(q, k, v, scale=1.0)
+    assert o.dtype == f8 and torch.all(o.float() == 88.0), o.float().unique()
+    # the same two keys as the first rows of a one-page cache
+    kc, vc = torch.zeros(1, 64, 1, 64), torch.zeros(1, 64, 1, 64)
+    kc[0, :2], vc[0, :2] = k[0].float().cpu(), v[0].float().cpu()
+    o_acc, lse_acc = fck.fmha_fwd_splitkv(q, dev(kc.to(f8)), dev(vc.to(f8)), 1, dev(torch.tensor([2], dtype=torch.int32)),
+                                          dev(torch.zeros(1, 1, dtype=torch.int32)), scale=1.0)
+    o = fck.fmha_fwd_splitkv_combine(lse_acc, o_acc, f8)
+    assert o.dtype == f8 and torch.all(o.float() == 88.0), o.float().unique()
