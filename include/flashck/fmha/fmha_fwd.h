@@ -27,6 +27,12 @@ namespace flashck {
 
 namespace naive {
 
+/* One e4m3 byte (OCP encoding): the element type that selects the all-fp8 roles (Q, K, V, P and O in e4m3,
+ * FCK_DTYPE_FP8) in the functions below, where the C ABI has kernels for them. */
+struct fp8_e4m3 {
+    unsigned char bits;
+};
+
 namespace fmha_detail {
 
 template <typename T>
@@ -38,6 +44,10 @@ struct DTypeOf<_Float16> {
 template <>
 struct DTypeOf<unsigned short> {
     static constexpr int32_t value = FCK_DTYPE_BF16;
+};
+template <>
+struct DTypeOf<fp8_e4m3> {
+    static constexpr int32_t value = FCK_DTYPE_FP8;
 };
 #if defined(__clang__)
 template <>

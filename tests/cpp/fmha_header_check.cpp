@@ -50,6 +50,8 @@ int main()
     const int bad = run<_Float16>() + run<unsigned short>();
     static_assert(flashck::naive::fmha_detail::DTypeOf<_Float16>::value == FCK_DTYPE_FP16, "fp16 id");
     static_assert(flashck::naive::fmha_detail::DTypeOf<unsigned short>::value == FCK_DTYPE_BF16, "bf16 id");
+    static_assert(flashck::naive::fmha_detail::DTypeOf<flashck::naive::fp8_e4m3>::value == FCK_DTYPE_FP8 && sizeof(flashck::naive::fp8_e4m3) == 1,
+                  "e4m3 id, one byte per element");
     std::printf(bad ? "FAILED: %d checks\n" : "OK\n", bad);
     return bad != 0;
 }
