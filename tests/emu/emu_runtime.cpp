@@ -2,6 +2,8 @@
 #include "emu_runtime.h"
 
 #include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
 #include <sys/mman.h>
 
 #include <vector>
@@ -90,9 +92,16 @@ void schedule()
         if (from >= 0) emu_switch(save, g.main_sp);
         return;
     }
-    int next = from;
+    // Fibers take turns in thread order, or in the opposite order with EMU_ORDER=reverse: between two barriers the
+    // waves of a workgroup then run last to first, so a wave that reads what an earlier wave wrote without a barrier in
+    // between - which the forward order lets pass - sees the poison instead.
+    static const bool reverse = [] {
+        const char* e = getenv("EMU_ORDER");
+        return e && strcmp(e, "reverse") == 0;
+    }();
+    int next = from < 0 && reverse ? 0 : from;
     do {
-        next = (next + 1) % g.n;
+        next = reverse ? (next + g.n - 1) % g.n : (next + 1) % g.n;
     } while (g.fibers[next].done);
     if (next == from) return;
     g.running = next;

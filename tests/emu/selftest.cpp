@@ -95,7 +95,26 @@ __global__ void async_kernel(const uint32_t* src, uint32_t* out)
     if (w == 0) wait_vm<0>();
 }
 
+// A missing barrier: each of two waves writes its number + 1 into its own LDS word and reads the other wave's word with
+// no barrier in between.  Whichever wave runs first sees the poison the emulator fills LDS with; the other one gets away
+// with the race.  out[w] = what wave w read.
+__global__ void race_kernel(uint32_t* out)
+{
+    FCK_DYNAMIC_LDS(smem);
+    uint32_t* lds = reinterpret_cast<uint32_t*>(smem);
+    const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (l == 0) {
+        lds[w] = (uint32_t)w + 1u;
+        out[w] = lds[w ^ 1];
+    }
+}
+
 extern "C" {
+__attribute__((visibility("default"))) int emu_selftest_race(uint32_t* out)
+{
+    hipLaunchKernelGGL(race_kernel, dim3(1), dim3(128), 8, nullptr, out);
+    return (int)hipGetLastError();
+}
 __attribute__((visibility("default"))) int emu_selftest_mfma(int shape, const uint16_t* a, const uint16_t* b, float* d)
 {
     if (shape == 0) hipLaunchKernelGGL((mfma_kernel<32, 16>), dim3(1), dim3(64), 0, nullptr, a, b, d);

@@ -67,3 +67,25 @@ def test_a_read_without_the_wait_sees_stale_lds(emu):
     assert torch.equal(out[:256], src[:256]) and (out[256:] == stale).all()         # the newest request may still be in flight
     assert emu.emu_selftest_async(2, _p(src), _p(out)) == 0
     assert (out == stale).all()
+
+
+_RACE = """
+import ctypes, sys, torch
+emu = ctypes.CDLL(sys.argv[1])
+out = torch.zeros(2, dtype=torch.int32)
+assert emu.emu_selftest_race(ctypes.c_void_p(out.data_ptr())) == 0
+print(out[0].item(), out[1].item())
+"""
+
+
+@pytest.mark.parametrize("order", ["forward", "reverse"])
+def test_the_wave_that_runs_first_sees_a_missing_barrier(order):
+    """Waves run first to last between barriers, last to first with EMU_ORDER=reverse: of two waves that read each other's
+    LDS word without a barrier, the one that runs first reads the poison (-1), the other one the value (wave number + 1).
+    A kernel that passes under both orders has no such read in either direction."""
+    import subprocess
+    import build_emu
+    env = dict(os.environ, EMU_ORDER=order)
+    r = subprocess.run([sys.executable, "-c", _RACE, build_emu.build()], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert r.stdout.split() == (["-1", "1"] if order == "forward" else ["2", "-1"]), r.stdout
