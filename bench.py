@@ -149,7 +149,7 @@ def bench_decode(args, torch, fmha, gen, which):
         scales = dict(k_descale=0.0625, v_descale=0.0625)
         w["k_cache"] = (w["k_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
         w["v_cache"] = (w["v_cache"].float() / 0.0625).to(torch.float8_e4m3fn)
-        name += " [Q, K, V, P, O fp8 e4m3]" if all_fp8 else " [K/V cache fp8 e4m3]"
+        name = name.replace("(bf16)", "(e4m3 in and out, bf16 matrix instructions)") if all_fp8 else name + " [K/V cache fp8 e4m3]"
     pools = [(w["k_cache"].to(dev), w["v_cache"].to(dev))]
     for _ in range(args.copies - 1):
         pools.append((pools[0][0].clone(), pools[0][1].clone()))
@@ -215,8 +215,9 @@ def bench_prefill(args, torch, fmha, gen, d, steps, warmup, variant=0, alibi=Fal
     flops = gen.prefill_flops(w["lens"], 32, d, dv or d)
     nbytes = gen.prefill_bytes(w["lens"], 32, 8, d, dv or d)
     ms = wall / steps * 1e3
-    tag = (f" (v_head_dim {dv})" if dv else "") + (" + ALiBi" if alibi else "") + (" [Q, K, V, P, O fp8 e4m3]" if all_fp8 else " [K/V cache fp8 e4m3]" if kv_fp8 else "") + (f" [tile variant {variant}]" if variant else "")
-    return dict(name=f"varlen causal batch prefill: 16 seqs L~U[128,8192] Hq32/Hk8 D{d} paged P=128 (bf16)" + tag,
+    tag = (f" (v_head_dim {dv})" if dv else "") + (" + ALiBi" if alibi else "") + (" [K/V cache fp8 e4m3]" if kv_fp8 and not all_fp8 else "") + (f" [tile variant {variant}]" if variant else "")
+    kind = "e4m3 in and out, bf16 matrix instructions" if all_fp8 else "bf16"
+    return dict(name=f"varlen causal batch prefill: 16 seqs L~U[128,8192] Hq32/Hk8 D{d} paged P=128 ({kind})" + tag,
                 ms_per_step=ms, flops=flops, bytes=nbytes, tflops=flops / (ms * 1e-3) / 1e12, kernel_ms=kern_ms,
                 kernel_tflops=flops / (kern_ms * 1e-3) / 1e12, total_q=sum(w["lens"]), kernel=kernel)
 
