@@ -155,3 +155,135 @@ def test_random_prefill(fmha, orc, seed):
             ro = orc.fmha_fwd(qb, kc, vc, seqlen_k=sl, block_table=bt, **common, **okw)
     kernel = _lib.load().fck_fmha_last_kernel().decode()
     assert_close(o, ro, ATOL[dtype], what + " [" + kernel + "]")
+
+
+def _pool_bits(t):
+    return t.contiguous().view(torch.uint8 if t.dtype == F8 else torch.int16).cpu()
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_appendkv(fmha, orc, seed):
+    """Whole pools and the rotated q compared bit for bit: appended rows as the oracle writes them, every other byte
+    (NaN fill of unused slots included) untouched."""
+    r = random.Random(9000 + seed)
+    g = torch.Generator().manual_seed(9000 + seed)
+    dtype = r.choice([torch.bfloat16, torch.float16])
+    B = r.randint(1, 5)
+    hk = r.choice([1, 2, 3, 4])
+    hq = hk * r.choice([1, 2, 4])
+    fp8 = r.random() < 0.3
+    d = r.choice([64, 128, 256] if fp8 else [32, 64, 96, 128, 192, 256])
+    dv = d if fp8 or r.random() < 0.7 else r.choice([64, 128])
+    page = r.choice([1, 16, 48, 64, 128])
+    rope_mode = r.choice([0, 1, 2, 2])
+    rotary_dim = r.choice([d, d // 2, 16, d - 16])
+    has_mask = r.random() < 0.7
+    with_q = r.random() < 0.8
+    lens = [r.randint(1, 400) for _ in range(B)]
+    new = [r.randint(1, 9) for _ in range(B)]
+    uniform = r.random() < 0.3   # [B, n, H, D] inputs without cu_seqlens
+    if uniform:
+        new = [new[0]] * B
+    cap = [l + n for l, n in zip(lens, new)]
+    kv = gen.paged_kv(lens, hk, d, dtype, g, page, capacity=cap, dv=dv if dv != d else None)
+    total = sum(new)
+    cu = torch.tensor([0] + list(torch.tensor(new).cumsum(0)), dtype=torch.int32)
+    q = gen.randn((total, hq, d), dtype, g) if with_q else None
+    knew, vnew = gen.randn((total, hk, d), dtype, g), gen.randn((total, hk, dv), dtype, g)
+    cos, sin = gen.rotary_tables(max(cap) + 1, rotary_dim, dtype) if rope_mode else (None, None)
+    what = (f"seed {seed}: {dtype} B={B} Hq{hq if with_q else 0}/Hk{hk} d=({d},{dv}) P={page} rope={rope_mode}/{rotary_dim} has_mask={has_mask} "
+            f"lens={lens} new={new} uniform={uniform} fp8={fp8}")
+    print(what, flush=True)
+    scales = {}
+    if fp8:
+        scales = dict(k_descale=r.choice([0.02, 0.05]), v_descale=r.choice([0.01, 0.03]))
+        fill = lambda t: torch.full(t.shape, 0x55, dtype=torch.uint8).view(F8)
+        kc0, vc0 = fill(kv["k_cache"]), fill(kv["v_cache"])
+    else:
+        kc0, vc0 = kv["k_cache"], kv["v_cache"]
+    dq, kc, vc = dev(q), dev(kc0), dev(vc0)
+    if uniform:
+        n = new[0]
+        shape = lambda t, h, dd: None if t is None else dev(t.view(B, n, h, dd))
+        fmha.fmha_fwd_appendkv(shape(q, hq, d), kc, vc, shape(knew, hk, d), shape(vnew, hk, dv), dev(kv["seqlen_k"]), rotary_cos=dev(cos),
+                               rotary_sin=dev(sin), rope_mode=rope_mode, has_mask=has_mask, block_table=dev(kv["block_table"]), **scales)
+        dq = None  # the view above was copied to the device on its own: compare that copy
+        if with_q:
+            dq = shape(q, hq, d)
+            kc, vc = dev(kc0), dev(vc0)
+            fmha.fmha_fwd_appendkv(dq, kc, vc, shape(knew, hk, d), shape(vnew, hk, dv), dev(kv["seqlen_k"]), rotary_cos=dev(cos),
+                                   rotary_sin=dev(sin), rope_mode=rope_mode, has_mask=has_mask, block_table=dev(kv["block_table"]), **scales)
+    else:
+        fmha.fmha_fwd_appendkv(dq, kc, vc, dev(knew), dev(vnew), dev(kv["seqlen_k"]), cu_seqlens_knew=dev(cu), max_seqlen_knew=max(new),
+                               rotary_cos=dev(cos), rotary_sin=dev(sin), rope_mode=rope_mode, has_mask=has_mask,
+                               block_table=dev(kv["block_table"]), **scales)
+    rq = q.clone() if with_q else None
+    rkc, rvc = kc0.clone(), vc0.clone()
+    orc.appendkv(rq, rkc, rvc, knew, vnew, kv["seqlen_k"], cu, cos=cos, sin=sin, rope_mode=rope_mode, has_mask=has_mask,
+                 block_table=kv["block_table"], **scales)
+    for name, a, b in (("k_cache", kc, rkc), ("v_cache", vc, rvc)) + ((("q", dq.view(total, hq, d), rq),) if with_q else ()):
+        bad = (_pool_bits(a) != _pool_bits(b)).nonzero()
+        assert bad.numel() == 0, f"{what}: {name}: {bad.shape[0]} elements differ, first at {bad[0].tolist()}"
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_decode_group_mode_bias_and_cache_rows(fmha, orc, seed):
+    """What test_random_decode leaves out: packed queries of ragged length (group mode) over a packed or paged K/V, an
+    elementwise bias of every rank, and a batch cache addressed through cache_batch_idx."""
+    r = random.Random(13000 + seed)
+    g = torch.Generator().manual_seed(13000 + seed)
+    dtype = r.choice([torch.bfloat16, torch.float16])
+    B = r.randint(1, 4)
+    hk = r.choice([1, 2, 4])
+    ratio = r.choice([1, 2, 4])
+    hq = hk * ratio
+    d = r.choice([64, 128, 256])
+    ns = r.randint(1, 4)
+    mask_type, window = _mask(r)
+    layout = r.choice(["group_packed", "group_paged", "batch_rows"])
+    lens_k = [r.randint(1, 300) for _ in range(B)]
+    common = dict(scale=1.0 / math.sqrt(d), mask_type=mask_type, window=window)
+    if layout == "batch_rows":
+        sq = r.choice([1, 2, 4])
+        rows, slots = max(lens_k) + r.randint(0, 9), B + r.randint(0, 2)
+        idx = torch.tensor(r.sample(range(slots), B), dtype=torch.int32)
+        k, v = gen.randn((slots, rows, hk, d), dtype, g), gen.randn((slots, rows, hk, d), dtype, g)
+        q = gen.randn((B, sq, hq, d), dtype, g)
+        sl = torch.tensor(lens_k, dtype=torch.int32)
+        bias_rows, group, min_cols = sq, False, rows   # a batch cache: a bias row spans the cache's rows
+        dkw = dict(seqlen_k=dev(sl), cache_batch_idx=dev(idx))
+        okw = dict(seqlen_k=sl, cache_batch_idx=idx)
+        ckw, ockw = {}, {}
+    else:
+        lens_q = [r.randint(1, 6) for _ in range(B)]
+        cq = torch.tensor([0] + list(torch.tensor(lens_q).cumsum(0)), dtype=torch.int32)
+        q = gen.randn((sum(lens_q), hq, d), dtype, g)
+        bias_rows, group, min_cols = sum(lens_q), True, max(lens_k)
+        if layout == "group_packed":
+            ck = torch.tensor([0] + list(torch.tensor(lens_k).cumsum(0)), dtype=torch.int32)
+            k, v = gen.randn((sum(lens_k), hk, d), dtype, g), gen.randn((sum(lens_k), hk, d), dtype, g)
+            dkw = dict(cu_seqlens_q=dev(cq), cu_seqlens_k=dev(ck), max_seqlen_q=max(lens_q))
+            okw = dict(seqstart_q=cq, seqstart_k=ck)
+        else:
+            kv = gen.paged_kv(lens_k, hk, d, dtype, g, r.choice([16, 48, 64, 128]))
+            k, v = kv["k_cache"], kv["v_cache"]
+            dkw = dict(cu_seqlens_q=dev(cq), max_seqlen_q=max(lens_q), seqlen_k=dev(kv["seqlen_k"]), block_table=dev(kv["block_table"]))
+            okw = dict(seqstart_q=cq, seqlen_k=kv["seqlen_k"], block_table=kv["block_table"])
+        ckw, ockw = dict(cu_seqlens_q=dev(cq), max_seqlen_q=max(lens_q)), dict(seqstart_q=cq)
+    rank = r.choice([None, 0, 1, 2])
+    if rank is not None:
+        cols = min_cols + r.choice([0, 0, 5])
+        shape = (1 if rank == 0 else hq, bias_rows, cols) if group else (B if rank == 2 else 1, 1 if rank == 0 else hq, bias_rows, cols)
+        bias = (gen.randn(shape, dtype, g) * 1.5).contiguous()
+        dkw["bias"], okw["bias"] = dev(bias), bias
+        if r.random() < 0.3:
+            dkw["logits_soft_cap"] = okw["logits_soft_cap"] = 3.0
+    what = f"seed {seed}: {layout} {dtype} B={B} Hq{hq}/Hk{hk} d={d} lens_k={lens_k} ns={ns} mask={mask_type}{window} bias rank {rank}"
+    print(what, flush=True)
+    o_acc, lse_acc = fmha.fmha_fwd_splitkv(dev(q), dev(k), dev(v), ns, **common, **dkw)
+    kernel = _lib.load().fck_fmha_last_kernel().decode()
+    o = fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, dtype, **ckw)
+    assert_close(o, orc.fmha_fwd(q, k, v, **common, **okw), ATOL[dtype], what + " [" + kernel + "]")
+    ra, rl = orc.fmha_splitkv(q, k, v, ns, **common, **okw)
+    assert_lse_close(lse_acc, rl, 2e-3, what + " lse_acc")
+    assert_close(o_acc, ra, ATOL[dtype], what + " o_acc")
