@@ -171,3 +171,67 @@ def test_what_the_roles_do_not_cover_is_refused(fmha):
     Kc, Vc = dev(_q8(kv["k_cache"], KD)), dev(_q8(kv["v_cache"], VD))
     with pytest.raises(NotImplementedError):                # the one-launch entry point has no e4m3 kernels
         fmha.fmha_fwd_splitkv_fused(Q[:, :1], Kc, Vc, 2, seqlen_k=dev(kv["seqlen_k"]), block_table=dev(kv["block_table"]))
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_problems(fmha, orc, seed):
+    """Seeded random problems with e4m3 q / k / v through split-KV + combine and the prefill addressings."""
+    import random
+    r = random.Random(17000 + seed)
+    g = torch.Generator().manual_seed(17000 + seed)
+    B = r.randint(1, 4)
+    hk = r.choice([1, 2, 4])
+    hq = hk * r.choice([1, 2, 4, 8])
+    d = r.choice([64, 128, 128, 256])
+    page = r.choice([16, 48, 64, 128])
+    path = r.choice(["decode", "decode", "page_list", "block_table", "dense_varlen"])
+    mask_type, left, right = r.choice([(0, -1, -1), (2, -1, 0), (2, -1, 0), (1, -1, 0), (2, 30, 0), (1, 5, 5)])
+    kw = dict(scale=QS / math.sqrt(d), k_descale=KD, v_descale=VD, mask_type=mask_type, window=(left, right))
+    extra = {}
+    pick = r.random()
+    if pick < 0.2:
+        extra["alibi_slopes"] = torch.tensor([r.uniform(0.0, 0.05) for _ in range(hq)], dtype=torch.float32)
+    elif pick < 0.35:
+        extra["logits_soft_cap"] = r.choice([2.0, 20.0])
+    dextra = {k: dev(v) for k, v in extra.items()}
+    if path == "decode":
+        sq, ns = r.choice([1, 1, 2, 4]), r.randint(1, 4)
+        lens = [r.randint(1, 700) for _ in range(B)]
+        what = f"seed {seed}: decode B={B} Hq{hq}/Hk{hk} sq={sq} d={d} P={page} lens={lens} ns={ns} mask={mask_type}({left},{right}) {sorted(extra)}"
+        print(what, flush=True)
+        kv = gen.paged_kv(lens, hk, d, torch.bfloat16, g, page)
+        Q, K, V = _q8(torch.randn(B, sq, hq, d, generator=g), QS), _q8(kv["k_cache"], KD), _q8(kv["v_cache"], VD)
+        o_acc, lse_acc = fmha.fmha_fwd_splitkv(dev(Q), dev(K), dev(V), ns, seqlen_k=dev(kv["seqlen_k"]), block_table=dev(kv["block_table"]),
+                                               **kw, **dextra)
+        o = fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, F8)
+        okw = dict(seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], **kw, **extra)
+    else:
+        top = r.choice([20, 140, 260])
+        lens_q = [r.randint(1, top) for _ in range(B)]
+        lens_k = [n + r.choice([0, 1, 90]) for n in lens_q]
+        what = f"seed {seed}: {path} B={B} Hq{hq}/Hk{hk} d={d} P={page} lens_q={lens_q} lens_k={lens_k} mask={mask_type}({left},{right}) {sorted(extra)}"
+        print(what, flush=True)
+        cq = torch.tensor([0] + list(torch.tensor(lens_q).cumsum(0)), dtype=torch.int32)
+        Q = _q8(torch.randn(sum(lens_q), hq, d, generator=g), QS)
+        if path == "dense_varlen":
+            ck = torch.tensor([0] + list(torch.tensor(lens_k).cumsum(0)), dtype=torch.int32)
+            K, V = _q8(torch.randn(sum(lens_k), hk, d, generator=g), KD), _q8(torch.randn(sum(lens_k), hk, d, generator=g), VD)
+            o = fmha.fmha_fwd_varlen(dev(Q), dev(K), dev(V), dev(cq), dev(ck), max(lens_q), **kw, **dextra)
+            okw = dict(seqstart_q=cq, seqstart_k=ck, **kw, **extra)
+        else:
+            kv = gen.paged_kv(lens_k, hk, d, torch.bfloat16, g, page)
+            K, V = _q8(kv["k_cache"], KD), _q8(kv["v_cache"], VD)
+            bt, sl = kv["block_table"], kv["seqlen_k"]
+            if path == "page_list":
+                n_pages = [(n + page - 1) // page for n in lens_k]
+                indptr = torch.tensor([0] + list(torch.tensor(n_pages).cumsum(0)), dtype=torch.int32)
+                indices = torch.cat([bt[b, :n_pages[b]] for b in range(B)]).contiguous()
+                last = torch.tensor([n - (p - 1) * page for n, p in zip(lens_k, n_pages)], dtype=torch.int32)
+                o = fmha.fmha_batch_prefill(dev(Q), dev(K), dev(V), dev(cq), dev(indptr), dev(indices), dev(last), max_seqlen_q=max(lens_q),
+                                            **kw, **dextra)
+                okw = dict(seqstart_q=cq, kv_indptr=indptr, kv_page_indices=indices, kv_last_page_lens=last, **kw, **extra)
+            else:
+                o = fmha.fmha_fwd_pagedkv(dev(Q), dev(K), dev(V), dev(sl), dev(bt), cu_seqlens_q=dev(cq), max_seqlen_q=max(lens_q), **kw, **dextra)
+                okw = dict(seqstart_q=cq, seqlen_k=sl, block_table=bt, **kw, **extra)
+    assert o.dtype == F8 and "all_fp8" in _last_kernel(), _last_kernel()
+    assert_fp8_roles_close(o, orc.fmha_fwd(Q, K, V, **okw), _fine(orc, Q, K, V, **okw), what)
