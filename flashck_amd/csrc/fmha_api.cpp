@@ -246,6 +246,9 @@ int fck_fmha_num_splits_heuristic(int64_t batch, int64_t hq, int64_t hk, int64_t
 {
     (void)head_dim;
     if (batch <= 0 || hq <= 0 || hk <= 0 || sq <= 0 || max_sk <= 0) return 1;
+    // sizes no launch could have (the products below must stay inside 64 bits and away from zero)
+    constexpr int64_t kMax = (int64_t)1 << 24;
+    if (batch > kMax || hq > kMax || hk > hq || sq > kMax || num_cu > kMax) return 1;
     if (num_cu <= 0) num_cu = cu_count();
     // One workgroup streams one split of one KV head for 16..64 packed rows (query index x head-in-group).
     const int64_t g = hq / hk;

@@ -90,6 +90,10 @@ def test_workspace_bytes_and_heuristic():
     assert fmha.num_splits_heuristic(1, 8, 8, 1, 200, 128, 256) == 1
     for args in [(1, 8, 1, 1, 10 ** 6, 128, 256), (32, 32, 8, 1, 4096, 128, 256)]:
         assert 1 <= fmha.num_splits_heuristic(*args) <= 128
+    # sizes no launch could have answer 1 (batch * kv heads used to wrap to zero here, and the next line divided by it)
+    assert lib.fck_fmha_num_splits_heuristic(1 << 31, 2, 1 << 62, 96, (1 << 31) - 1, 1, 1 << 31) == 1
+    assert lib.fck_fmha_num_splits_heuristic(4, 2, 8, 1, 4096, 128, 256) == 1      # more KV heads than query heads
+    assert lib.fck_fmha_num_splits_heuristic(1 << 40, 8, 8, 1, 4096, 128, 256) == 1
 
 
 def test_python_validation_mirrors_reference_errors():
