@@ -38,8 +38,19 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
+// The kernels keep counts and lengths in 32 bits: a larger argument would be cut down to some other, valid-looking
+// problem, so it is refused instead.
+template <typename... T>
+int check_fit32(T... v)
+{
+    if (((v > (int64_t)INT32_MAX || v < (int64_t)INT32_MIN) || ...))
+        return fail(FCK_ERR_INVALID_ARGUMENT, "a count, length or stride argument is beyond 32 bits");
+    return FCK_OK;
+}
+
 int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, int32_t dtype)
 {
+    if (int rc = check_fit32(batch, hq, hk, d, dv)) return rc;
     if (dtype != FCK_DTYPE_FP16 && dtype != FCK_DTYPE_BF16 && dtype != FCK_DTYPE_FP8)
         return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT8 (1, e4m3), FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
     if (dtype == FCK_DTYPE_FP8 && (d != dv || (d != 64 && d != 128 && d != 256)))
@@ -284,6 +295,7 @@ static int splitkv_setup(fck::SplitKvArgs& a, bool& uniform, int& rows_max, cons
     if (group && seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "group mode: seqlen_q must carry total_q (workspace row count)");
     if (q_max_seq_len <= 0) q_max_seq_len = seqlen_q;
     if (q_max_seq_len <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "q_max_seq_len must be positive");
+    if (int rc = check_fit32(seqlen_q, seqlen_k, q_max_seq_len, max_num_page_blocks, page_block_size, q_max_seq_len * (hq / hk))) return rc;
 
     a = fck::SplitKvArgs{};
     a.q = q;
@@ -513,6 +525,7 @@ int fck_fmha_fwd_splitkv_combine(const void* lse_acc, const void* o_acc, void* o
         return fail(FCK_ERR_UNSUPPORTED, "dtype %d: only FLOAT8 (1, e4m3), FLOAT16 (3) and BFLOAT16 (4) have kernels", dtype);
     if (!lse_acc || !o_acc || !o) return fail(FCK_ERR_INVALID_ARGUMENT, "lse_acc, o_acc and o must not be null");
     if (batch <= 0 || hq <= 0 || seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch, q_num_heads and seqlen_q must be positive");
+    if (int rc = check_fit32(batch, seqlen_q, hq, dv, num_splits)) return rc;
     if (dv < 8 || dv > 256 || dv % 8) return fail(FCK_ERR_UNSUPPORTED, "v_head_dim %ld: a multiple of 8 in [8, 256]", (long)dv);
     if (num_splits < 1 || num_splits > 128) return fail(FCK_ERR_INVALID_ARGUMENT, "num_splits %ld out of range [1,128]", (long)num_splits);
     if (!aligned16(o_acc) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_acc and o must be 16-byte aligned");
@@ -573,6 +586,7 @@ int fck_fmha_fwd_appendkv_attrs(void* q, void* k_cache, void* v_cache, const voi
     if (batch <= 0 || hk <= 0 || d <= 0 || dv <= 0 || (q && hq <= 0)) return fail(FCK_ERR_INVALID_ARGUMENT, "sizes must be positive");
     if (d % 2 || dv % 2) return fail(FCK_ERR_INVALID_ARGUMENT, "head dims must be even");
     if (seqlen_knew <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "seqlen_knew (largest number of new tokens of a sequence) must be positive");
+    if (int rc = check_fit32(batch, hq, hk, d, dv, seqlen_knew, rotary_dim, batch_stride_block_table, page_block_size, seqlen_k_cache)) return rc;
     if (rope_mode < 0 || rope_mode > 2) return fail(FCK_ERR_INVALID_ARGUMENT, "rope_mode %d out of range [0,2]", rope_mode);
     if (rope_mode != FCK_ROPE_NONE) {
         if (!rotary_cos || !rotary_sin) return fail(FCK_ERR_INVALID_ARGUMENT, "rotary tables must not be null when rope_mode != NONE");
@@ -708,6 +722,7 @@ int fck_fmha_fwd_attrs(const void* q, const void* k, const void* v, const void* 
     if (int rc = check_common(batch, hq, hk, d, dv, dtype)) return rc;
     if (int rc = check_mask(mask_type)) return rc;
     if (!q || !k || !v || !o) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v and o must not be null");
+    if (int rc = check_fit32(seqlen_q, seqlen_k, q_max_seq_len)) return rc;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k, v and o must be 16-byte aligned");
     if (!(scale > 0.f) || !std::isfinite(scale)) return fail(FCK_ERR_INVALID_ARGUMENT, "scale must be positive and finite");
     if ((seqstart_q == nullptr) != (seqstart_k == nullptr)) return fail(FCK_ERR_INVALID_ARGUMENT, "group mode needs both seqstart_q and seqstart_k");
@@ -766,6 +781,7 @@ int fck_fmha_batch_prefill_attrs(const void* q, const void* k_cache, const void*
         return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, seqstart_q, kv_indptr and kv_page_indices must not be null");
     if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache and o must be 16-byte aligned");
     if (page_block_size <= 0 || num_total_pages <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "page_block_size and num_total_pages must be positive");
+    if (int rc = check_fit32(page_block_size, num_total_pages, q_max_seq_len)) return rc;
     if (!(scale > 0.f) || !std::isfinite(scale)) return fail(FCK_ERR_INVALID_ARGUMENT, "scale must be positive and finite");
     fck::PrefillArgs a{};
     a.q = q;
@@ -818,6 +834,7 @@ int fck_fmha_fwd_pagedkv_attrs(const void* q, const void* k_cache, const void* v
         return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, seqlen_k and block_table must not be null");
     if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(o)) return fail(FCK_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache and o must be 16-byte aligned");
     if (page_block_size <= 0 || batch_stride_block_table <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "page_block_size and batch_stride_block_table must be positive");
+    if (int rc = check_fit32(page_block_size, batch_stride_block_table, seqlen_q, q_max_seq_len)) return rc;
     if (!(scale > 0.f) || !std::isfinite(scale)) return fail(FCK_ERR_INVALID_ARGUMENT, "scale must be positive and finite");
     if (!seqstart_q && seqlen_q <= 0) return fail(FCK_ERR_INVALID_ARGUMENT, "batch mode needs seqlen_q > 0");
     fck::PrefillArgs a{};

@@ -242,3 +242,26 @@ def test_fp8_roles_are_validated_before_any_launch():
     # an unknown dtype still names the ones there are
     rc = lib.fck_fmha_fwd_splitkv_combine(p, p, p, None, 1, 1, 2, 64, 1, 2, 9, None)
     assert rc == -2 and b"FLOAT8" in lib.fck_last_error()
+
+
+def test_sizes_beyond_32_bits_are_refused_not_truncated():
+    """2^32 + 1 sequences must not run as 1 sequence: counts, lengths and strides the kernels keep in 32 bits are range-checked."""
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    big = (1 << 32) + 1
+    msg = b"beyond 32 bits"
+    assert lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, big, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, 4, None) == -1 and msg in lib.fck_last_error()
+    assert lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, big, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, 4, None) == -1 and msg in lib.fck_last_error()
+    assert lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, big, 0.125, -1, -1, 0, 4, None) == -1 and msg in lib.fck_last_error()
+    rc = lib.fck_fmha_fwd_splitkv(p, p, p, None, p, p, None, None, None, None, None, 1, 1, big, 2, 2, 64, 64, 1, 2, 0, 0, 0.125, -1, -1, 0, 4, None)
+    assert rc == -1 and msg in lib.fck_last_error()
+    rc = lib.fck_fmha_fwd_splitkv(p, p, p, None, p, p, None, None, p, p, None, 1, 1, 0, 2, 2, 64, 64, 1, 2, 4, big, 0.125, -1, -1, 0, 4, None)
+    assert rc == -1 and msg in lib.fck_last_error()
+    assert lib.fck_fmha_fwd_splitkv_combine(p, p, p, None, 1, big, 2, 64, 1, 2, 4, None) == -1 and msg in lib.fck_last_error()
+    rc = lib.fck_fmha_fwd_appendkv(None, p, p, p, p, p, None, big, None, None, 0, 0, 0, p, 4, 16, None, 0, 1, 2, 2, 64, 64, 4, None)
+    assert rc == -1 and msg in lib.fck_last_error()
+    rc = lib.fck_fmha_batch_prefill(p, p, p, p, p, p, p, None, big, 16, 1, 2, 2, 64, 64, 8, 0.125, -1, 0, 2, 4, None)
+    assert rc == -1 and msg in lib.fck_last_error()
+    rc = lib.fck_fmha_fwd_pagedkv(p, p, p, p, None, p, p, big, 16, 1, 8, 2, 2, 64, 64, 8, 0.125, -1, 0, 2, 4, None)
+    assert rc == -1 and msg in lib.fck_last_error()
