@@ -389,7 +389,13 @@ static hipError_t launch_d(const PrefillArgs& a, bool uniform, hipStream_t st)
         if (uniform) return launch_with_lds<prefill_kernel<T, D, true, true>>(grid, dim3(256), lds, st, a);
         return launch_with_lds<prefill_kernel<T, D, false, true>>(grid, dim3(256), lds, st, a);
     }
-    if (uniform) return launch_with_lds<prefill_kernel<T, D, true>>(grid, dim3(256), lds, st, a);
+    if (uniform) {
+        // plain calls over tile-aligned pages at head dim 256 belong to the direct-to-LDS kernel: no instantiation here
+        if constexpr (D == 256)
+            return hipErrorInvalidValue;
+        else
+            return launch_with_lds<prefill_kernel<T, D, true>>(grid, dim3(256), lds, st, a);
+    }
     return launch_with_lds<prefill_kernel<T, D, false>>(grid, dim3(256), lds, st, a);
 }
 

@@ -226,6 +226,20 @@ uint64_t ballot(bool p)
     return m;
 }
 
+void note_launch(const char* tag)
+{
+    static const char* path = getenv("EMU_COVERAGE");
+    if (!path) return;
+    static std::vector<const char*> seen;  // type_info names: one address per instantiation
+    for (const char* s : seen)
+        if (s == tag) return;
+    seen.push_back(tag);
+    if (FILE* f = fopen(path, "a")) {
+        fprintf(f, "%s\n", tag);
+        fclose(f);
+    }
+}
+
 void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>& body)
 {
     const int n = (int)(block.x * block.y * block.z);

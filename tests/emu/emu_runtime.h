@@ -17,6 +17,7 @@
 
 #include <cmath>
 #include <functional>
+#include <typeinfo>
 #include <type_traits>
 
 // ---- language keywords ------------------------------------------------------------------------------------------------
@@ -68,6 +69,11 @@ extern thread_local Lane* cur;
 // last launch failed (a kernel broke a rule of the emulator: see emu_runtime.cpp); cleared by the read
 hipError_t take_error();
 void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>& body);
+// EMU_COVERAGE=<file>: the first launch of every kernel instantiation in a process appends the mangled name of
+// KernelTag<&kernel<...>> to the file (c++filt turns it into the instantiation): what a test run has launched.
+template <auto Kernel>
+struct KernelTag {};
+void note_launch(const char* tag);
 // How the asynchronous global -> LDS copies are modelled.  true (default): a copy lands at the LAST moment the
 // program allows - when the lane that requested it waits for its outstanding copies to drop below the copy's place in
 // the queue, or when the lane ends - so a read that is not covered by the proper wait sees stale (poisoned) LDS and the
@@ -95,7 +101,8 @@ inline T lane_value(const char* all, int lane)
 }  // namespace emu
 
 inline hipError_t hipGetLastError() { return emu::take_error(); }
-#define hipLaunchKernelGGL(kern, grid, block, lds, stream, ...) emu::launch((grid), (block), (lds), [=]() { kern(__VA_ARGS__); })
+#define hipLaunchKernelGGL(kern, grid, block, lds, stream, ...) \
+    (emu::note_launch(typeid(emu::KernelTag<kern>).name()), emu::launch((grid), (block), (lds), [=]() { kern(__VA_ARGS__); }))
 
 #define threadIdx (emu::cur->tid)
 #define blockIdx (emu::cur->bid)

@@ -25,7 +25,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(HERE, "emu"))
 
 GPU_MODULES = ["test_gpu_decode", "test_gpu_combine", "test_gpu_appendkv", "test_gpu_prefill", "test_gpu_prefill_grid",
-               "test_gpu_score_mods", "test_gpu_head_dims", "test_gpu_step", "test_zr_random_shapes", "test_zt_prefill_variants", "test_zu_fast_kernel_mods", "test_zv_fp8_cache", "test_zw_validate", "test_zx_fp8_roles", "test_zy_flash_ck_module",
+               "test_gpu_score_mods", "test_gpu_head_dims", "test_gpu_step", "test_zr_random_shapes", "test_zs_every_instantiation", "test_zt_prefill_variants", "test_zu_fast_kernel_mods", "test_zv_fp8_cache", "test_zw_validate", "test_zx_fp8_roles", "test_zy_flash_ck_module",
                "test_zz_no_alloc"]
 # need a real device: HIP graph capture
 NEEDS_DEVICE = {"test_decode_captured_in_a_graph"}
