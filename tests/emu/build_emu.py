@@ -21,6 +21,15 @@ FLAGS = ["-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-fvisibility=hidden",
          "-Wall", "-Wno-unused-function", "-Wno-unused-variable", "-Wno-unused-but-set-variable", "-Wno-unknown-pragmas"]
 
 
+# FCK_EMU_GCOV=1: a second build with line and branch counters (clang --coverage, read with gcov), in its own directory
+# and library, for finding the kernel and C-ABI code no test executes: tests/emu/line_coverage.py
+GCOV = os.environ.get("FCK_EMU_GCOV") == "1"
+if GCOV:
+    OBJ = os.path.join(HERE, "build_gcov")
+    LIB = os.path.join(HERE, "libflashck_fmha_emu_gcov.so")
+    FLAGS = FLAGS + ["--coverage"]
+
+
 def _compile(path):
     obj = os.path.join(OBJ, os.path.splitext(os.path.basename(path))[0] + ".o")
     if os.path.exists(obj) and os.path.getmtime(obj) > max(
@@ -58,7 +67,7 @@ def _build():
         objs = list(ex.map(_compile, paths))
     if os.path.exists(LIB) and os.path.getmtime(LIB) >= max(os.path.getmtime(o) for o in objs):
         return LIB
-    r = subprocess.run([CXX, "-shared", "-fPIC", "-o", LIB + ".tmp"] + objs + ["-lpthread", "-lm"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    r = subprocess.run([CXX, "-shared", "-fPIC", "-o", LIB + ".tmp"] + objs + ["-lpthread", "-lm"] + (["--coverage"] if GCOV else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"emulator link failed:\n{r.stdout[-4000:]}")
     os.replace(LIB + ".tmp", LIB)

@@ -127,3 +127,27 @@ def test_fp8_cache_argument_checks(fmha):
         fmha.fmha_fwd_appendkv(*args, k_descale=0.0, **kw)
     with pytest.raises(TypeError):   # one cache fp8, the other 16-bit
         fmha.fmha_fwd_appendkv(None, kc, dev(w["v_cache"]), *args[3:], **kw)
+
+
+@pytest.mark.parametrize("with_idx", [True, False])
+def test_appendkv_fp8_into_a_batch_cache(fmha, orc, with_idx):
+    """A non-paged fp8 cache [slots, rows, Hk, D], addressed directly or through cache_batch_idx; packed, ragged new tokens."""
+    g = torch.Generator().manual_seed(19)
+    B, hk, hq, d, rows = 3, 2, 4, 64, 48
+    new = [4, 1, 7]
+    cu = torch.tensor([0, 4, 5, 12], dtype=torch.int32)
+    knew, vnew = gen.randn((12, hk, d), torch.bfloat16, g), gen.randn((12, hk, d), torch.bfloat16, g)
+    q = gen.randn((12, hq, d), torch.bfloat16, g)
+    sl = torch.tensor([0, 36, 17], dtype=torch.int32)
+    idx = torch.tensor([3, 1, 4], dtype=torch.int32) if with_idx else None
+    cos, sin = gen.rotary_tables(rows + 1, d, torch.bfloat16)
+    slots = 5 if with_idx else B
+    q_ref, kc_ref, vc_ref = q.clone(), _fp8_pool((slots, rows, hk, d)), _fp8_pool((slots, rows, hk, d))
+    orc.appendkv(q_ref, kc_ref, vc_ref, knew, vnew, sl, cu, cos, sin, rope_mode=2, has_mask=True, cache_batch_idx=idx, k_descale=0.04, v_descale=0.02)
+    qd, kcd, vcd = dev(q.clone()), dev(_fp8_pool((slots, rows, hk, d))), dev(_fp8_pool((slots, rows, hk, d)))
+    fmha.fmha_fwd_appendkv(qd, kcd, vcd, dev(knew), dev(vnew), dev(sl), cu_seqlens_knew=dev(cu), max_seqlen_knew=max(new), rotary_cos=dev(cos),
+                           rotary_sin=dev(sin), rope_mode=2, cache_batch_idx=dev(idx), k_descale=0.04, v_descale=0.02)
+    _bytes_equal(kcd, kc_ref, "k_cache")
+    _bytes_equal(vcd, vc_ref, "v_cache")
+    assert_bits_equal(qd, q_ref, "q")
+    assert (kc_ref.view(torch.uint8) != 0x55).any(), "the append must have written something"
