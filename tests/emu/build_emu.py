@@ -28,6 +28,23 @@ if GCOV:
     OBJ = os.path.join(HERE, "build_gcov")
     LIB = os.path.join(HERE, "libflashck_fmha_emu_gcov.so")
     FLAGS = FLAGS + ["--coverage"]
+# FCK_EMU_UBSAN=1: a build with the undefined-behaviour sanitizer (indexing past a fixed-size array, misaligned vector
+# accesses, signed overflow, shifts out of range); a finding aborts the process with a report
+UBSAN = os.environ.get("FCK_EMU_UBSAN") == "1"
+if UBSAN:
+    OBJ = os.path.join(HERE, "build_ubsan")
+    LIB = os.path.join(HERE, "libflashck_fmha_emu_ubsan.so")
+    FLAGS = FLAGS + ["-fsanitize=bounds,alignment,signed-integer-overflow,shift,null,integer-divide-by-zero", "-fno-sanitize-recover=all"]
+
+
+def _sanitizer_dir():
+    """where clang keeps its shared sanitizer runtimes"""
+    r = subprocess.run([CXX, "-print-file-name=libclang_rt.ubsan_standalone-x86_64.so"], stdout=subprocess.PIPE, text=True)
+    path = r.stdout.strip()
+    if not os.path.isabs(path):   # not in the default place: search the resource directory
+        res = subprocess.run([CXX, "-print-resource-dir"], stdout=subprocess.PIPE, text=True).stdout.strip()
+        path = os.path.join(res, "lib", "linux", "libclang_rt.ubsan_standalone-x86_64.so")
+    return os.path.dirname(path)
 
 
 def _compile(path):
@@ -67,7 +84,8 @@ def _build():
         objs = list(ex.map(_compile, paths))
     if os.path.exists(LIB) and os.path.getmtime(LIB) >= max(os.path.getmtime(o) for o in objs):
         return LIB
-    r = subprocess.run([CXX, "-shared", "-fPIC", "-o", LIB + ".tmp"] + objs + ["-lpthread", "-lm"] + (["--coverage"] if GCOV else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    r = subprocess.run([CXX, "-shared", "-fPIC", "-o", LIB + ".tmp"] + objs + ["-lpthread", "-lm"] + (["--coverage"] if GCOV else []) +
+                       (["-fsanitize=undefined", "-shared-libsan", "-Wl,-rpath," + _sanitizer_dir()] if UBSAN else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"emulator link failed:\n{r.stdout[-4000:]}")
     os.replace(LIB + ".tmp", LIB)
