@@ -7,6 +7,7 @@ arguments (q, k, v, seqstart_q, seqstart_k, seqlen_k); the module style follows 
 the same kernels: prefill over a paged cache and the append -> split-KV -> combine decode step, with the workspace kept
 between steps.
 """
+import math
 from typing import Optional, Tuple
 
 import torch
@@ -66,10 +67,14 @@ class Attention(torch.nn.Module):
 
 class PagedAttention(torch.nn.Module):
     """Causal attention over a paged KV cache [num_pages, page_size, Hk, D]: `prefill` for whole prompts already in the
-    cache, `decode_step` for appending new tokens and attending from them."""
+    cache, `decode_step` for appending new tokens and attending from them.  The caches may be torch.float8_e4m3fn with the
+    static per-tensor scales k_descale / v_descale (value = descale * stored; the reference's is_static_quant,
+    core/profiling/attention/fmha_fwd_split_kv/fmha_fwd_split_kv_problem.h:79): decode_step then quantises what it
+    appends and both calls dequantise what they read."""
 
     def __init__(self, q_num_heads: int, kv_num_heads: int, qk_head_dim: int, v_head_dim: Optional[int] = None,
-                 scale: float = 0.0, window_left: int = -1, rope_mode: int = fmha.ROPE_NONE, num_splits: int = 0):
+                 scale: float = 0.0, window_left: int = -1, rope_mode: int = fmha.ROPE_NONE, num_splits: int = 0,
+                 k_descale: float = 1.0, v_descale: float = 1.0):
         super().__init__()
         v_head_dim = qk_head_dim if v_head_dim is None else v_head_dim
         _check_heads(q_num_heads, kv_num_heads, qk_head_dim, v_head_dim)
@@ -83,6 +88,9 @@ class PagedAttention(torch.nn.Module):
         self.window_left = int(window_left)
         self.rope_mode = rope_mode
         self.num_splits = int(num_splits)
+        if not (k_descale > 0.0 and v_descale > 0.0 and math.isfinite(k_descale) and math.isfinite(v_descale)):
+            raise ValueError("k_descale and v_descale must be positive and finite")
+        self.k_descale, self.v_descale = float(k_descale), float(v_descale)
         self.workspace = fmha.DecodeWorkspace()
 
     def _check_cache(self, q, k_cache, v_cache):
@@ -102,12 +110,12 @@ class PagedAttention(torch.nn.Module):
         if kv_indptr is not None:
             return fmha.fmha_batch_prefill(q, k_cache, v_cache, cu_seqlens_q, kv_indptr, kv_page_indices, kv_last_page_lens,
                                            max_seqlen_q=max_seqlen_q, scale=self.scale, mask_type=fmha.MASK_BOTTOM_RIGHT,
-                                           window=window)
+                                           window=window, k_descale=self.k_descale, v_descale=self.v_descale)
         if block_table is None or seqlen_k is None:
             raise ValueError("prefill needs either kv_indptr/kv_page_indices or block_table/seqlen_k")
         return fmha.fmha_fwd_pagedkv(q, k_cache, v_cache, seqlen_k, block_table, cu_seqlens_q=cu_seqlens_q,
                                      max_seqlen_q=max_seqlen_q, scale=self.scale, mask_type=fmha.MASK_BOTTOM_RIGHT,
-                                     window=window)
+                                     window=window, k_descale=self.k_descale, v_descale=self.v_descale)
 
     def decode_step(self, q, knew, vnew, k_cache, v_cache, seqlen_k, block_table, *, cu_seqlens_knew=None,
                     max_seqlen_knew: int = 0, rotary_cos=None, rotary_sin=None, max_seqlen_k: int = 0, out=None):
@@ -118,9 +126,10 @@ class PagedAttention(torch.nn.Module):
                                      cu_seqlens_knew=cu_seqlens_knew, max_seqlen_knew=max_seqlen_knew,
                                      rotary_cos=rotary_cos, rotary_sin=rotary_sin, rope_mode=self.rope_mode,
                                      num_splits=self.num_splits, max_seqlen_k=max_seqlen_k, scale=self.scale,
-                                     window_left=self.window_left, workspace=self.workspace, out=out)
+                                     window_left=self.window_left, workspace=self.workspace, out=out,
+                                     k_descale=self.k_descale, v_descale=self.v_descale)
 
     def extra_repr(self) -> str:
         return (f"q_num_heads={self.q_num_heads}, kv_num_heads={self.kv_num_heads}, qk_head_dim={self.qk_head_dim}, "
                 f"v_head_dim={self.v_head_dim}, scale={self.scale}, window_left={self.window_left}, "
-                f"rope_mode={self.rope_mode}, num_splits={self.num_splits}")
+                f"rope_mode={self.rope_mode}, num_splits={self.num_splits}, k_descale={self.k_descale}, v_descale={self.v_descale}")

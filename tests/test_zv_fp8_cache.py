@@ -151,3 +151,32 @@ def test_appendkv_fp8_into_a_batch_cache(fmha, orc, with_idx):
     _bytes_equal(vcd, vc_ref, "v_cache")
     assert_bits_equal(qd, q_ref, "q")
     assert (kc_ref.view(torch.uint8) != 0x55).any(), "the append must have written something"
+
+
+def test_paged_attention_module_over_fp8_cache(fmha, orc):
+    """The module carries the static scales: a decode step (quantising append + attention) and a prefill over the same
+    quantised cache, against the oracle's chain."""
+    from flashck_amd.nn import PagedAttention
+    w = gen.workload_appendkv_decode(seed=11, batch=3, hq=8, hk=2, head_dim=128, min_len=20, max_len=400, max_new=3, page_size=64)
+    kd, vd = 0.03, 0.025
+    k8, v8 = _quantised(w, kd, vd)
+    m = PagedAttention(8, 2, 128, rope_mode=2, num_splits=2, k_descale=kd, v_descale=vd)
+    assert "k_descale=0.03" in repr(m)
+    q, kc, vc = dev(w["q"]), dev(k8), dev(v8)
+    o, sl_new = m.decode_step(q, dev(w["knew"]), dev(w["vnew"]), kc, vc, dev(w["seqlen_k"]), dev(w["block_table"]),
+                              cu_seqlens_knew=dev(w["cu_seqlens_knew"]), max_seqlen_knew=w["max_new"], rotary_cos=dev(w["rotary_cos"]),
+                              rotary_sin=dev(w["rotary_sin"]))
+    q_ref, k_ref, v_ref = w["q"].clone(), k8.clone(), v8.clone()
+    orc.appendkv(q_ref, k_ref, v_ref, w["knew"], w["vnew"], w["seqlen_k"], w["cu_seqlens_knew"], cos=w["rotary_cos"], sin=w["rotary_sin"],
+                 rope_mode=2, has_mask=True, block_table=w["block_table"], k_descale=kd, v_descale=vd)
+    ref_len = w["seqlen_k"] + torch.tensor(w["new"], dtype=torch.int32)
+    okw = dict(seqstart_q=w["cu_seqlens_knew"], seqlen_k=ref_len, block_table=w["block_table"], mask_type=2, window=(-1, 0),
+               k_descale=kd, v_descale=vd)
+    _bytes_equal(kc, k_ref, "k_cache after the step")
+    assert torch.equal(sl_new.cpu(), ref_len)
+    assert_close(o, orc.fmha_fwd(q_ref, k_ref, v_ref, **okw), 2e-2, "module decode step")
+    # prefill of the same (new) tokens as a prompt over the grown cache: same problem through the prefill kernels
+    o2 = m.prefill(q, kc, vc, dev(w["cu_seqlens_knew"]), seqlen_k=sl_new, block_table=dev(w["block_table"]), max_seqlen_q=w["max_new"])
+    assert_close(o2, orc.fmha_fwd(q_ref, k_ref, v_ref, **okw), 2e-2, "module prefill")
+    with pytest.raises(ValueError, match="positive and finite"):
+        PagedAttention(8, 2, 128, k_descale=0.0)
