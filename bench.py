@@ -142,7 +142,7 @@ def bench_decode(args, torch, fmha, gen, which):
     kv_fp8 = getattr(args, "kv_fp8", False) or all_fp8
     scales = {}
     if all_fp8:
-        q = (q.float() / 0.0625).to(torch.float8_e4m3fn)
+        q = (w["q"].float() / 0.0625).to(torch.float8_e4m3fn).to(dev)  # cast on the host, as the tests do
         w["scale"] = w["scale"] * 0.0625
     if kv_fp8:
         # unit-variance data: a static scale of 1/16 keeps it well inside the e4m3 range (+-448)
