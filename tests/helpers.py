@@ -67,7 +67,7 @@ def fp8_step(x):
 def assert_fp8_close(a, b, what="", atol=FP8_ATOL, outliers=0.0):
     """a: e4m3 result; b: e4m3 or wider reference."""
     assert a.dtype == torch.float8_e4m3fn, f"{what}: result is {a.dtype}"
-    a, b = a.float().cpu(), b.float().cpu()
+    a, b = a.cpu().float(), b.cpu().float()   # e4m3 is widened on the host
     assert a.shape == b.shape, f"{what}: shape {a.shape} vs {b.shape}"
     assert torch.isfinite(a).all(), f"{what}: non-finite values in the result"
     diff = (a - b).abs()
@@ -84,6 +84,6 @@ def assert_fp8_roles_close(o, oracle8, fine, what="", atol=FP8_ATOL):
     reference's order); fine: the oracle on the same e4m3 inputs with 16-bit roles for Q, P and O (times o_scale)."""
     assert_fp8_close(o, fine, what + " vs the 16-bit roles", atol, outliers=1e-4)
     assert_fp8_close(o, oracle8, what + " vs the fp8 roles of the oracle", atol, outliers=1e-3)
-    f = fine.float().cpu()
-    e_dev, e_orc = (o.float().cpu() - f).abs().mean().item(), (oracle8.float().cpu() - f).abs().mean().item()
+    f = fine.cpu().float()
+    e_dev, e_orc = (o.cpu().float() - f).abs().mean().item(), (oracle8.cpu().float() - f).abs().mean().item()
     assert e_dev <= 1.05 * e_orc + 1e-6, f"{what}: mean error to the 16-bit roles {e_dev:.5f}, the oracle's fp8 roles have {e_orc:.5f}"
