@@ -279,6 +279,7 @@ struct ScoreMod {
     int32_t bias_type;  // 0 none, 1 elementwise, 2 ALiBi
     float soft_cap;     // > 0: on
     float scale;        // the softmax scale in natural units (the soft cap is not linear, so it cannot be folded)
+    int32_t bias_f32;   // elementwise: the bias holds fp32 (the e4m3 type roles), strides in floats; 0: the data type T
     __host__ __device__ bool active() const { return bias_type != 0 || soft_cap > 0.f; }
 };
 
@@ -306,6 +307,7 @@ __device__ __forceinline__ float fast_tanh(float x)
 template <typename T>
 struct RowMod {
     const uint16_t* bias_row;  // elementwise: row (b, h, i) of the bias
+    const float* bias_row32;   // the same when the bias holds fp32 (then bias_row is null)
     float slope;               // ALiBi: signed slope (positive for VERTICAL, negative otherwise)
     int32_t zero;              // ALiBi: column of distance 0 (unused for VERTICAL)
     int32_t mode;
@@ -323,13 +325,17 @@ struct RowMod {
         last_key = sk - 1;
         if (m.cols > 0 && m.cols - 1 < last_key) last_key = (int32_t)(m.cols - 1);
         bias_row = nullptr;
+        bias_row32 = nullptr;
         slope = 0.f;
         zero = 0;
         mode = alibi_mode(mask_type, wl, wr);
         if (m.bias_type == 1) {
             const int64_t brow = (group ? first_row : 0) + i;
-            bias_row = reinterpret_cast<const uint16_t*>(m.bias) + (group ? 0 : (int64_t)b * m.batch_stride) + (int64_t)h * m.head_stride +
-                       brow * m.row_stride;
+            const int64_t off = (group ? 0 : (int64_t)b * m.batch_stride) + (int64_t)h * m.head_stride + brow * m.row_stride;
+            if (m.bias_f32)
+                bias_row32 = reinterpret_cast<const float*>(m.bias) + off;
+            else
+                bias_row = reinterpret_cast<const uint16_t*>(m.bias) + off;
         } else if (m.bias_type == 2) {
             const float sl = reinterpret_cast<const float*>(m.bias)[(int64_t)b * m.batch_stride + h];
             slope = mode == kAlibiVertical ? sl : -sl;
@@ -341,7 +347,8 @@ struct RowMod {
         float x = qk * scale;
         if (cap > 0.f) x = cap * fast_tanh(x * cap_rcp);
         if (bias_type == 1) {
-            x += T::to_f32(bias_row[min(max(key, 0), last_key)]);
+            const int col = min(max(key, 0), last_key);
+            x += bias_row32 ? bias_row32[col] : T::to_f32(bias_row[col]);
         } else if (bias_type == 2) {
             const int dist = mode == kAlibiVertical ? key : abs(zero - key);
             x = __builtin_fmaf(slope, (float)dist, x);

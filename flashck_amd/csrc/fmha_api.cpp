@@ -70,13 +70,14 @@ int check_common(int64_t batch, int64_t hq, int64_t hk, int64_t d, int64_t dv, i
 int compute_dtype(int32_t dtype) { return dtype == FCK_DTYPE_FP8 ? FCK_DTYPE_BF16 : dtype; }
 
 // The all-fp8 roles of a call (dtype FLOAT8): what the K/V descales do not cover.  `at` may be null.
-int fill_q8(int32_t& q8, float* o_scale, const fck::ScoreMod& mod, const fck_fmha_attrs* at, int32_t dtype)
+int fill_q8(int32_t& q8, float* o_scale, fck::ScoreMod& mod, const fck_fmha_attrs* at, int32_t dtype)
 {
     q8 = 0;
     if (o_scale) *o_scale = 1.f;
+    mod.bias_f32 = 0;
     if (dtype != FCK_DTYPE_FP8) return FCK_OK;
-    // BiasDataType of the fp8 roles is float (fmha_common_jinja.h:157-171): no kernel reads such a bias
-    if (mod.bias_type == FCK_BIAS_ELEMENTWISE) return fail(FCK_ERR_UNSUPPORTED, "an elementwise bias with e4m3 queries has no kernel");
+    // BiasDataType of the fp8 roles is float (fmha_common_jinja.h:157-171): an elementwise bias holds fp32, strides in floats
+    if (mod.bias_type == FCK_BIAS_ELEMENTWISE) mod.bias_f32 = 1;
     const float os = at && at->o_scale != 0.f ? at->o_scale : 1.f;
     if (!(os > 0.f) || !std::isfinite(os)) return fail(FCK_ERR_INVALID_ARGUMENT, "o_scale must be positive and finite (0: 1)");
     if (!o_scale && os != 1.f)

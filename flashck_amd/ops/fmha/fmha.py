@@ -130,7 +130,7 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
 
     o_scale (float8_e4m3fn queries on the dense / paged / page-list prefill calls): the output is
     saturate(o_scale * o) in e4m3.
-    bias (elementwise, BiasEnum ELEMENTWISE_BIAS): q's dtype, last dim contiguous; batch mode [1|B, 1|Hq, sq, >= sk],
+    bias (elementwise, BiasEnum ELEMENTWISE_BIAS): q's dtype (float32 for float8_e4m3fn queries), last dim contiguous; batch mode [1|B, 1|Hq, sq, >= sk],
     group mode [1|Hq, total_q, >= max sk]; size-1 dims are shared (the reference's rank 0 / 1 / 2).
     alibi_slopes (ALIBI): fp32 [Hq] or [B, Hq].  logits_soft_cap > 0: s = cap * tanh(scale * qk / cap).
     Returns (pointer argument, object to keep alive until the call has been made)."""
@@ -165,8 +165,9 @@ def _attrs(q, bias, alibi_slopes, logits_soft_cap, group, batch, rows, min_cols,
             raise TypeError(f"Expected bias to be a torch.Tensor, got {type(bias)}")
         if _REQUIRE_GPU_TENSORS and not bias.is_cuda:
             raise ValueError(f"bias must live on the GPU (got device {bias.device})")
-        if bias.dtype != q.dtype:
-            raise TypeError(f"bias must have q's dtype {q.dtype}, got {bias.dtype}")
+        want = torch.float32 if q.dtype == torch.float8_e4m3fn else q.dtype   # BiasDataType of the e4m3 roles is float
+        if bias.dtype != want:
+            raise TypeError(f"bias must have dtype {want} for {q.dtype} queries, got {bias.dtype}")
         if bias.dim() != (3 if group else 4) or bias.stride(-1) != 1:
             raise ValueError(f"bias must be {'[1|Hq, total_q, sk]' if group else '[1|B, 1|Hq, sq, sk]'} with a contiguous last dim, "
                              f"got shape {tuple(bias.shape)} strides {bias.stride()}")

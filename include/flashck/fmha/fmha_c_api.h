@@ -43,9 +43,9 @@ extern "C" {
  * e4m3 byte per element, P is rounded to e4m3 before the second product (scale_p = 1, as the reference passes it:
  * fmha_fwd_jinja.h:327), LSE and the split-KV partial results stay fp32.  k = k_descale * stored, v = v_descale * stored
  * as for an fp8 cache (a query scale belongs into `scale`); O = saturate(o_scale * o).  Needs qk_head_dim = v_head_dim in
- * {64, 128, 256}; no elementwise bias (its type would be fp32); not on fck_fmha_fwd_splitkv_fused / _appendkv.  The
- * products run on the bf16 matrix instructions (every e4m3 value is a bf16 value): the roles halve the memory traffic,
- * they do not double the matrix rate. */
+ * {64, 128, 256}; an elementwise bias holds fp32 for these roles (BiasDataType = float), strides in floats; not on
+ * fck_fmha_fwd_splitkv_fused / _appendkv.  The products run on the bf16 matrix instructions (every e4m3 value is a bf16
+ * value): the roles halve the memory traffic, they do not double the matrix rate. */
 #define FCK_DTYPE_FP8 1
 #define FCK_DTYPE_FP16 3
 #define FCK_DTYPE_BF16 4
@@ -77,7 +77,7 @@ extern "C" {
  * core/module/kernels/attention_kernels/fmha_common_jinja.h:157-171).
  *
  * Scores: x = scale * q.k;  x = cap * tanh(x / cap) when logits_soft_cap > 0;  x += bias;  then the mask.
- *   ELEMENTWISE_BIAS  T elements; (b, h, i, j) at bias[b * bias_batch_stride + h * bias_head_stride + i * bias_row_stride + j].
+ *   ELEMENTWISE_BIAS  T elements (fp32 when dtype is FCK_DTYPE_FP8); (b, h, i, j) at bias[b * bias_batch_stride + h * bias_head_stride + i * bias_row_stride + j].
  *                     The reference's rank 0 (1*1*s*s) is head and batch stride 0, rank 1 (1*h*s*s) batch stride 0,
  *                     rank 2 (b*h*s*s) neither.  Group mode: i counts packed query rows (seqstart_q[b] + local row)
  *                     and bias_batch_stride is not used.

@@ -314,7 +314,7 @@ static void attend_row(const fck_orc_problem* p, const void* q, const void* k, c
         float sv = acc * (p->scale * kd);
         if (p->logits_soft_cap > 0.f) sv = p->logits_soft_cap * tanhf(sv / p->logits_soft_cap);
         if (p->bias_type == 1) {
-            sv += ld(p->bias, bias_row + j, dt);
+            sv += dt == FCK_ORC_FP8 ? ((const float*)p->bias)[bias_row + j] : ld(p->bias, bias_row + j, dt); /* BiasDataType = float for fp8 */
         } else if (p->bias_type == 2) {
             /* Alibi::update (row major): VERTICAL adds slope * col; the two diagonal modes add -slope * |zero - col| with
                zero = row (top left) or row + sk - sq (bottom right: shift_right_down - shift_left_up = sk - sq) */
@@ -359,7 +359,6 @@ static int max_sk(const fck_orc_problem* p)
 static int check(const fck_orc_problem* p)
 {
     if (p->dtype != FCK_ORC_BF16 && p->dtype != FCK_ORC_FP16 && p->dtype != FCK_ORC_FP8) return -1;
-    if (p->dtype == FCK_ORC_FP8 && p->bias_type == 1) return -3; /* BiasDataType of the fp8 roles is float: not restated */
     if (p->hk <= 0 || p->hq % p->hk) return -2;
     return 0;
 }

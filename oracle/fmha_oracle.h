@@ -79,7 +79,7 @@ typedef struct {
     /* dtype FCK_ORC_FP8: the all-fp8 roles of FmhaFwdTypeConfig<fp8_t> (fmha_common_jinja.h:157-171): Q, K, V, P and O are
        e4m3 (K/V as with kv_dtype FCK_ORC_FP8, the descales apply).  P is cast to e4m3 before the second product
        (p_compute_element_func = scales{scale_p}, scale_p = 1 in the reference) and O = saturate(o_scale * o) (0 means 1;
-       the reference passes scale_o = 1).  ck_tile/ops/fmha/kernel/fmha_fwd_kernel.hpp:1529-1553. */
+       the reference passes scale_o = 1).  An elementwise bias holds fp32 (BiasDataType = float), strides in floats.  ck_tile/ops/fmha/kernel/fmha_fwd_kernel.hpp:1529-1553. */
     float o_scale;
 } fck_orc_problem;
 

@@ -164,7 +164,8 @@ def _problem(q, k, v, *, seqstart_q=None, seqstart_k=None, seqlen_k=None, block_
         p.o_scale = float(o_scale)
     assert bias is None or alibi_slopes is None, "one bias kind at a time"
     if bias is not None:
-        assert bias.dtype == q.dtype and bias.device.type == "cpu" and bias.stride(-1) == 1
+        want = torch.float32 if q.dtype == torch.float8_e4m3fn else q.dtype   # BiasDataType of the fp8 roles is float
+        assert bias.dtype == want and bias.device.type == "cpu" and bias.stride(-1) == 1
         group = seqstart_q is not None
         assert bias.dim() == (3 if group else 4)
         p.bias_type = 1

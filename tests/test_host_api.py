@@ -211,12 +211,6 @@ def test_fp8_roles_are_validated_before_any_launch():
     assert rc == -2 and b"e4m3" in lib.fck_last_error()
     rc = lib.fck_fmha_fwd(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 128, 64, 8, 0.125, -1, -1, 0, FP8, None)
     assert rc == -2 and b"e4m3" in lib.fck_last_error()
-    # an elementwise bias (it would be fp32 for these roles)
-    at = _lib.Attrs()
-    at.size = ctypes.sizeof(_lib.Attrs)
-    at.bias_type, at.bias, at.bias_row_stride, at.bias_cols = 1, p.value, 8, 8
-    rc = lib.fck_fmha_fwd_attrs(p, p, p, None, p, None, None, None, 1, 8, 8, 2, 2, 64, 64, 8, 0.125, -1, -1, 0, FP8, ctypes.byref(at), None)
-    assert rc == -2 and b"bias" in lib.fck_last_error()
     # scales
     at = _lib.Attrs()
     at.size = ctypes.sizeof(_lib.Attrs)

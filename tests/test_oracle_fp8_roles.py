@@ -124,8 +124,27 @@ def test_one_split_combine_equals_the_forward(orc):
     assert torch.equal(o.view(torch.uint8), o1.view(torch.uint8))
 
 
-def test_elementwise_bias_is_not_restated_for_fp8(orc):
+def test_elementwise_bias_is_float32(orc):
+    """BiasDataType of the fp8 roles is float: against the torch restatement with the bias added to the scores, for a
+    bias shared by all heads and batches, per head, and per batch and head."""
+    g = torch.Generator().manual_seed(8)
+    B, sq, sk, Hq, Hk, D = 2, 9, 40, 4, 2, 64
+    qs, kd, vd = 0.02, 0.025, 0.03
+    Q = _q8(torch.randn(B, sq, Hq, D, generator=g), qs)
+    K = _q8(torch.randn(B, sk, Hk, D, generator=g), kd)
+    V = _q8(torch.randn(B, sk, Hk, D, generator=g), vd)
+    scale = qs / math.sqrt(D)
+    for shape in ((1, 1, sq, sk), (1, Hq, sq, sk), (B, Hq, sq, sk + 2)):
+        bias = (torch.randn(*shape, generator=g) * 2).contiguous()
+        o = orc.fmha_fwd(Q, K, V, scale=scale, k_descale=kd, v_descale=vd, bias=bias)
+        qf = Q.float()
+        kf = (K.float() * kd).repeat_interleave(Hq // Hk, 2)
+        vf = (V.float() * vd).repeat_interleave(Hq // Hk, 2)
+        s_ = torch.einsum("bqhd,bkhd->bhqk", qf, kf) * scale + bias[..., :sk]
+        ref = torch.einsum("bhqk,bkhd->bqhd", s_.softmax(-1).to(F8).float(), vf).clamp(-448, 448).to(F8)
+        diff = (_codes(o) - _codes(ref)).abs()
+        assert diff.max().item() <= 1 and (diff == 0).float().mean().item() > 0.99, f"bias {shape}: {(diff != 0).sum().item()} codes differ"
+    # a bias in another type is refused by the wrapper
     import pytest
-    q, k, v = _two_key_case()
     with pytest.raises(AssertionError):
-        orc.fmha_fwd(q, k, v, scale=1.0, bias=torch.zeros(1, 1, 1, 2).to(F8))
+        orc.fmha_fwd(Q, K, V, scale=scale, bias=torch.zeros(1, 1, sq, sk).to(F8))

@@ -25,6 +25,12 @@ def _fine(orc, Q, K, V, o_scale=1.0, **kw):
     return orc.fmha_fwd(Q.float().to(torch.bfloat16), K, V, **kw).float() * o_scale
 
 
+def _fine_bias(orc, Q, K, V, bias, **kw):
+    """_fine with an elementwise bias: the 16-bit roles take the bias in their own type, so it is rounded to bf16 first
+    (2^-9 relative: far below an e4m3 step)"""
+    return orc.fmha_fwd(Q.float().to(torch.bfloat16), K, V, bias=bias.to(torch.bfloat16), **kw).float()
+
+
 def _last_kernel():
     return _lib.load().fck_fmha_last_kernel().decode()
 
@@ -160,7 +166,7 @@ def test_what_the_roles_do_not_cover_is_refused(fmha):
     g = torch.Generator().manual_seed(2)
     Q = dev(_q8(torch.randn(1, 4, 2, 128, generator=g), QS))
     K = dev(_q8(torch.randn(1, 40, 2, 128, generator=g), KD))
-    with pytest.raises((NotImplementedError, TypeError)):   # an elementwise bias would be fp32 for these roles
+    with pytest.raises(TypeError):                          # the elementwise bias of these roles is float32
         fmha.fmha_fwd(Q, K, K, bias=dev(torch.zeros(1, 1, 4, 40).to(F8)))
     with pytest.raises(NotImplementedError):                # stored head dims other than 64 / 128 / 256
         fmha.fmha_fwd(dev(_q8(torch.randn(1, 4, 2, 96, generator=g), QS)), dev(_q8(torch.randn(1, 40, 2, 96, generator=g), KD)),
@@ -235,3 +241,30 @@ def test_random_problems(fmha, orc, seed):
                 okw = dict(seqstart_q=cq, seqlen_k=sl, block_table=bt, **kw, **extra)
     assert o.dtype == F8 and "all_fp8" in _last_kernel(), _last_kernel()
     assert_fp8_roles_close(o, orc.fmha_fwd(Q, K, V, **okw), _fine(orc, Q, K, V, **okw), what)
+
+
+@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("rank", [0, 1, 2])
+def test_elementwise_bias_is_float32(fmha, orc, d, rank):
+    """BiasDataType of these roles is float: every rank, dense forward (batch mode) and paged split-KV + combine."""
+    g = torch.Generator().manual_seed(3 * d + rank)
+    B, sq, sk, Hq, Hk = 2, 140, 170, 4, 2
+    Q = _q8(torch.randn(B, sq, Hq, d, generator=g), QS)
+    K = _q8(torch.randn(B, sk, Hk, d, generator=g), KD)
+    V = _q8(torch.randn(B, sk, Hk, d, generator=g), VD)
+    bias = (torch.randn(B if rank == 2 else 1, 1 if rank == 0 else Hq, sq, sk + 3, generator=g) * 1.5).contiguous()
+    kw = dict(scale=QS / math.sqrt(d), k_descale=KD, v_descale=VD, mask_type=2, window=(-1, 0))
+    o = fmha.fmha_fwd(dev(Q), dev(K), dev(V), bias=dev(bias), **kw)
+    assert "all_fp8" in _last_kernel()
+    assert_fp8_roles_close(o, orc.fmha_fwd(Q, K, V, bias=bias, **kw), _fine_bias(orc, Q, K, V, bias, **kw), f"dense D={d} bias rank {rank}")
+    # decode: 3 queries per sequence over a paged cache
+    lens = [150, 40]
+    kv = gen.paged_kv(lens, Hk, d, torch.bfloat16, g, 64)
+    Kc, Vc = _q8(kv["k_cache"], KD), _q8(kv["v_cache"], VD)
+    Qd = _q8(torch.randn(B, 3, Hq, d, generator=g), QS)
+    bd = (torch.randn(B if rank == 2 else 1, 1 if rank == 0 else Hq, 3, max(lens), generator=g) * 1.5).contiguous()
+    okw = dict(seqlen_k=kv["seqlen_k"], block_table=kv["block_table"], **kw)
+    o_acc, lse_acc = fmha.fmha_fwd_splitkv(dev(Qd), dev(Kc), dev(Vc), 2, seqlen_k=dev(kv["seqlen_k"]), block_table=dev(kv["block_table"]),
+                                           bias=dev(bd), **kw)
+    o = fmha.fmha_fwd_splitkv_combine(lse_acc, o_acc, F8)
+    assert_fp8_roles_close(o, orc.fmha_fwd(Qd, Kc, Vc, bias=bd, **okw), _fine_bias(orc, Qd, Kc, Vc, bd, **okw), f"decode D={d} bias rank {rank}")
