@@ -27,6 +27,13 @@ struct Fiber {
 struct WaveState {
     int live, arrived;
     unsigned gen;
+    // global -> LDS instruction slots in flight through the wave's lanes (a lane's n-th request is slot n): how many lanes
+    // have passed each, and how many of them with a real request
+    unsigned char slot_lanes[1024], slot_real[1024];
+    int lanes0;                  // lanes the wave started with
+    unsigned max_requests;       // most requests any lane has made
+    unsigned ended_after[64];    // requests made by each lane that has ended
+    int n_ended;
     alignas(64) char buf[2][64][256];
 };
 
@@ -81,6 +88,19 @@ void fail(const char* what)
     }
 }
 
+// Instruction slot n of a wave is complete when every lane that gets that far has passed it: the lanes the wave started
+// with minus those that ended after fewer than n + 1 requests.  A complete slot must have had a real request.
+void close_slot(WaveState& w, unsigned n)
+{
+    int expected = w.lanes0;
+    for (int i = 0; i < w.n_ended; ++i)
+        if (w.ended_after[i] <= n) --expected;
+    const unsigned slot = n & 1023u;
+    if (w.slot_lanes[slot] == 0 || (int)w.slot_lanes[slot] < expected) return;
+    if (w.slot_real[slot] == 0) fail("a global -> LDS instruction with every lane of the wave masked off: the hardware would not issue it");
+    w.slot_lanes[slot] = w.slot_real[slot] = 0;
+}
+
 // run the next fiber that has not finished; back to the launcher when none is left
 void schedule()
 {
@@ -124,6 +144,8 @@ void fiber_exit()
     --g.live;
     WaveState& w = g.waves[f.lane.wave];
     --w.live;
+    if (w.n_ended < 64) w.ended_after[w.n_ended++] = f.lane.requests;
+    for (unsigned n = f.lane.requests; n < w.max_requests; ++n) close_slot(w, n);  // slots this lane will never reach
     if (w.arrived > 0 && w.arrived >= w.live) fail("a lane ended while other lanes of its wave wait in a cross-lane instruction");
     if (g.bar_arrived > 0 && g.bar_arrived >= g.live) {  // the hardware barrier does not wait for ended waves
         g.bar_arrived = 0;
@@ -193,6 +215,19 @@ bool late_loads()
 
 void request_copy(char* dst, const char* src)
 {
+    // The waits count INSTRUCTIONS per wave.  An instruction that every lane of a wave skips is not issued at all (the
+    // compiler branches around it when no lane is active), so the wave's count of outstanding copies would be one lower
+    // than the wait was written for, and an older copy could still be in flight behind it.  A kernel that masks lanes
+    // off (padded head dims) must therefore keep at least one lane on every instruction.
+    {
+        Lane& l = *cur;
+        WaveState& w = g.waves[l.wave];
+        const unsigned n = l.requests++;
+        if (l.requests > w.max_requests) w.max_requests = l.requests;
+        ++w.slot_lanes[n & 1023u];
+        if (dst) ++w.slot_real[n & 1023u];
+        close_slot(w, n);
+    }
     if (!late_loads()) {
         if (dst) memcpy(dst, src, 16);
         return;
@@ -271,6 +306,10 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
                     w.live = 0;
                     w.arrived = 0;
                     w.gen = 0;
+                    memset(w.slot_lanes, 0, sizeof(w.slot_lanes));
+                    memset(w.slot_real, 0, sizeof(w.slot_real));
+                    w.lanes0 = w.n_ended = 0;
+                    w.max_requests = 0;
                 }
                 for (int t = 0; t < n; ++t) {
                     Fiber& f = g.fibers[t];
@@ -281,8 +320,10 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
                     f.lane.lane = t & 63;
                     f.lane.wave = t >> 6;
                     f.lane.pending_head = f.lane.pending_count = 0;
+                    f.lane.requests = 0;
                     f.done = false;
                     ++g.waves[t >> 6].live;
+                    ++g.waves[t >> 6].lanes0;
                     // initial frame: six callee-saved registers, then the entry point as return address; the stack
                     // pointer is 8 modulo 16 when fiber_main starts, as after a call
                     uintptr_t top = (uintptr_t)(g.stacks + (size_t)(t + 1) * kStack) & ~(uintptr_t)15;

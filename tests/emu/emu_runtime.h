@@ -71,6 +71,7 @@ struct Lane {
     int lane, wave;
     PendingCopy pending[256];  // FIFO: vector-memory operations complete in order
     int pending_head, pending_count;
+    unsigned requests;  // global -> LDS requests this lane has made so far (real or masked)
 };
 extern thread_local Lane* cur;
 

@@ -109,7 +109,24 @@ __global__ void race_kernel(uint32_t* out)
     }
 }
 
+// A global -> LDS instruction that `real` lanes of the wave take part in and the others are masked off for.
+__global__ void masked_kernel(const uint32_t* src, int real)
+{
+    FCK_DYNAMIC_LDS(smem);
+    const int l = threadIdx.x & 63;
+    if (l < real)
+        load_to_lds(lds_address((char FCK_LDS*)smem), src, (uint32_t)l * 16u);
+    else
+        FCK_LOAD_TO_LDS_MASKED();
+    wait_vm<0>();
+}
+
 extern "C" {
+__attribute__((visibility("default"))) int emu_selftest_masked(const uint32_t* src, int real)
+{
+    hipLaunchKernelGGL(masked_kernel, dim3(1), dim3(64), 1024, nullptr, src, real);
+    return (int)hipGetLastError();
+}
 __attribute__((visibility("default"))) int emu_selftest_race(uint32_t* out)
 {
     hipLaunchKernelGGL(race_kernel, dim3(1), dim3(128), 8, nullptr, out);
